@@ -1,0 +1,267 @@
+/*
+ * C ABI of the MI355X (gfx950) data-tiled matmul microkernel library.
+ *
+ * The first group of entry points keeps the names, argument order, argument
+ * meaning, struct layouts and flag values of the reference CPU microkernels in
+ * runtime/src/iree/builtins/ukernel so that a caller of those can link against
+ * this library unchanged. The second group (prefix iree_uk_mi355x_) has no
+ * counterpart in the reference: it exposes what a GPU implementation needs in
+ * addition (device selection, stream-ordered launches).
+ *
+ * Pointer arguments may be host pointers or HIP device pointers. Classification
+ * looks only at `buffer + offset` (never at `buffer` itself, which the
+ * reference's own tests set to an address before the allocation), see
+ * iree_uk_mi355x_set_stream() for the rules.
+ *
+ * Everything here is plain C: no HIP or torch types appear in a signature.
+ */
+#ifndef IREE_UK_MI355X_H_
+#define IREE_UK_MI355X_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Signed 64-bit index type on 64-bit targets (reference: common.h:269-275). */
+typedef long long iree_uk_index_t;
+
+/*===--------------------------------------------------------------------===*/
+/* Flag values. Fixed by the reference compiler and runtime sharing them      */
+/* (reference: exported_bits.h:29-49, 56-66, 73-83).                          */
+/*===--------------------------------------------------------------------===*/
+
+#define IREE_UK_FLAG_MMT4D_TYPE_MASK 0xFF
+#define IREE_UK_FLAG_MMT4D_TYPE_NONE 0x00
+#define IREE_UK_FLAG_MMT4D_TYPE_F32F32F32 0x01
+#define IREE_UK_FLAG_MMT4D_TYPE_S8S8S32 0x02
+#define IREE_UK_FLAG_MMT4D_TYPE_F16F16F32 0x03
+#define IREE_UK_FLAG_MMT4D_TYPE_F16F16F16 0x04
+#define IREE_UK_FLAG_MMT4D_TYPE_BF16BF16F32 0x05
+#define IREE_UK_FLAG_MMT4D_TYPE_BF16BF16BF16 0x06
+#define IREE_UK_FLAG_MMT4D_TYPE_S16S16S32 0x07
+#define IREE_UK_FLAG_MMT4D_TYPE_S16U4S32 0x08
+#define IREE_UK_FLAG_MMT4D_TYPE_S16S8S32 0x09
+#define IREE_UK_FLAG_MMT4D_TYPE_S8S4S32 0x0A
+#define IREE_UK_FLAG_MMT4D_TYPE_END 0x0B
+#define IREE_UK_FLAG_MMT4D_ACCUMULATE 0x100
+#define IREE_UK_FLAG_MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION 0x200
+#define IREE_UK_FLAG_MMT4D_SKIP_INTERMEDIATE_ROUNDINGS 0x400
+#define IREE_UK_FLAG_MMT4D_INFO_HAVE_ARCHITECTURE_SPECIFIC_TILE_FUNCTION 0x1
+
+#define IREE_UK_FLAG_PACK_TYPE_MASK 0xFF
+#define IREE_UK_FLAG_PACK_TYPE_NONE 0x00
+#define IREE_UK_FLAG_PACK_TYPE_F32F32 0x01
+#define IREE_UK_FLAG_PACK_TYPE_I8I8 0x02
+#define IREE_UK_FLAG_PACK_TYPE_I32I32 0x03
+#define IREE_UK_FLAG_PACK_TYPE_F16F16 0x04
+#define IREE_UK_FLAG_PACK_TYPE_BF16BF16 0x05
+#define IREE_UK_FLAG_PACK_TRANSPOSE_INNER 0x100
+#define IREE_UK_FLAG_PACK_TRANSPOSE_OUTER 0x200
+
+#define IREE_UK_FLAG_UNPACK_TYPE_MASK 0xFF
+#define IREE_UK_FLAG_UNPACK_TYPE_NONE 0x00
+#define IREE_UK_FLAG_UNPACK_TYPE_F32F32 0x01
+#define IREE_UK_FLAG_UNPACK_TYPE_I32I32 0x03
+#define IREE_UK_FLAG_UNPACK_TYPE_F16F16 0x04
+#define IREE_UK_FLAG_UNPACK_TYPE_BF16BF16 0x05
+#define IREE_UK_FLAG_UNPACK_TRANSPOSE_INNER 0x100
+#define IREE_UK_FLAG_UNPACK_TRANSPOSE_OUTER 0x200
+
+#define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_MASK 0xFF
+#define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_LHS 0x01
+#define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_RHS 0x02
+#define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_RESULT 0x03
+#define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MASK 0xFF00
+#define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_F32F32F32 0x0100
+#define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_I8I8I32 0x0200
+#define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_F16F16F32 0x0300
+#define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_F16F16F16 0x0400
+#define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_BF16BF16F32 0x0500
+#define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_BF16BF16BF16 0x0600
+
+/*===--------------------------------------------------------------------===*/
+/* Parameter structs (field order and types are ABI).                         */
+/*===--------------------------------------------------------------------===*/
+
+/* reference: mmt4d_internal.h:14-32. Offsets and strides count ELEMENTS of the
+ * operand's type (4-bit elements included); M, N, K count tiles. Only the
+ * outermost dimension of each operand is strided. */
+typedef struct iree_uk_mmt4d_params_t {
+  const void* lhs_buffer;
+  iree_uk_index_t lhs_offset;
+  iree_uk_index_t lhs_stride0;
+  const void* rhs_buffer;
+  iree_uk_index_t rhs_offset;
+  iree_uk_index_t rhs_stride0;
+  void* out_buffer;
+  iree_uk_index_t out_offset;
+  iree_uk_index_t out_stride0;
+  iree_uk_index_t M;
+  iree_uk_index_t N;
+  iree_uk_index_t K;
+  int32_t M0;
+  int32_t N0;
+  int32_t K0;
+  uint32_t flags;
+  const uint64_t* cpu_data;
+} iree_uk_mmt4d_params_t;
+
+/* reference: pack_internal.h:12-30. */
+typedef struct iree_uk_pack_params_t {
+  const void* in_buffer;
+  iree_uk_index_t in_offset;
+  iree_uk_index_t in_stride0;
+  iree_uk_index_t in_stride1;
+  void* out_buffer;
+  iree_uk_index_t out_offset;
+  iree_uk_index_t out_stride0;
+  iree_uk_index_t out_stride1;
+  iree_uk_index_t in_size0;
+  iree_uk_index_t in_size1;
+  iree_uk_index_t out_size0;
+  iree_uk_index_t out_size1;
+  iree_uk_index_t out_size2;
+  iree_uk_index_t out_size3;
+  uint64_t padding_value;
+  uint32_t flags;
+  const uint64_t* cpu_data;
+} iree_uk_pack_params_t;
+
+/* reference: unpack_internal.h:12-29. */
+typedef struct iree_uk_unpack_params_t {
+  const void* in_buffer;
+  iree_uk_index_t in_offset;
+  iree_uk_index_t in_stride0;
+  iree_uk_index_t in_stride1;
+  void* out_buffer;
+  iree_uk_index_t out_offset;
+  iree_uk_index_t out_stride0;
+  iree_uk_index_t out_stride1;
+  iree_uk_index_t in_size0;
+  iree_uk_index_t in_size1;
+  iree_uk_index_t in_size2;
+  iree_uk_index_t in_size3;
+  iree_uk_index_t out_size0;
+  iree_uk_index_t out_size1;
+  uint32_t flags;
+  const uint64_t* cpu_data;
+} iree_uk_unpack_params_t;
+
+/* reference: query_tile_sizes.h:17-27. */
+typedef struct iree_uk_query_tile_sizes_2d_params_t {
+  uint32_t flags;
+  iree_uk_index_t size0;
+  iree_uk_index_t size1;
+  const uint64_t* cpu_data;
+} iree_uk_query_tile_sizes_2d_params_t;
+
+typedef struct iree_uk_query_tile_sizes_2d_out_params_t {
+  iree_uk_index_t tile_size0;
+  iree_uk_index_t tile_size1;
+} iree_uk_query_tile_sizes_2d_out_params_t;
+
+/*===--------------------------------------------------------------------===*/
+/* Entry points shared with the reference.                                    */
+/*===--------------------------------------------------------------------===*/
+
+/* out[M,N,M0,N0] (+)= lhs[M,K,M0,K0] * rhs[N,K,N0,K0]^T.
+ * Replaces: mmt4d.h:14-21 (flat form), mmt4d_internal.h:35 (struct form),
+ * implemented by mmt4d.c:115-177. `cpu_data` is accepted and ignored (may be
+ * NULL). IREE_UK_FLAG_MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION is accepted;
+ * tile shapes without an MFMA kernel always run on the generic GPU kernel. */
+void iree_uk_mmt4d(const void* lhs_buffer, iree_uk_index_t lhs_offset,
+                   iree_uk_index_t lhs_stride0, const void* rhs_buffer,
+                   iree_uk_index_t rhs_offset, iree_uk_index_t rhs_stride0,
+                   void* out_buffer, iree_uk_index_t out_offset,
+                   iree_uk_index_t out_stride0, iree_uk_index_t M,
+                   iree_uk_index_t N, iree_uk_index_t K, int32_t M0, int32_t N0,
+                   int32_t K0, uint32_t flags, const uint64_t* cpu_data);
+void iree_uk_mmt4d_p(const iree_uk_mmt4d_params_t* params);
+
+/* Bit 0 is set iff a kernel specialised for (type, M0, N0, K0) exists, here an
+ * MFMA or bandwidth-tuned kernel rather than the one-thread-per-element one.
+ * Replaces: mmt4d.h:25-27, mmt4d_internal.h:40, mmt4d.c:143-149,179-185. */
+uint32_t iree_uk_mmt4d_info(int32_t M0, int32_t N0, int32_t K0, uint32_t flags,
+                            const uint64_t* cpu_data);
+uint32_t iree_uk_mmt4d_info_p(const iree_uk_mmt4d_params_t* params);
+
+/* 2-D -> 4-D tiled copy with padding and optional inner/outer transposes.
+ * Replaces: pack.h:26-34, pack_internal.h:32, pack.c:315-352. */
+void iree_uk_pack(const void* in_buffer, iree_uk_index_t in_offset,
+                  iree_uk_index_t in_stride0, iree_uk_index_t in_stride1,
+                  void* out_buffer, iree_uk_index_t out_offset,
+                  iree_uk_index_t out_stride0, iree_uk_index_t out_stride1,
+                  iree_uk_index_t in_size0, iree_uk_index_t in_size1,
+                  iree_uk_index_t out_size0, iree_uk_index_t out_size1,
+                  iree_uk_index_t out_size2, iree_uk_index_t out_size3,
+                  uint64_t padding_value, uint32_t flags,
+                  const uint64_t* cpu_data);
+void iree_uk_pack_p(const iree_uk_pack_params_t* params);
+
+/* Inverse of pack; writes only the out_size0 x out_size1 logical region.
+ * Replaces: unpack.h:17-25, unpack_internal.h:31, unpack.c:249-285. */
+void iree_uk_unpack(const void* in_buffer, iree_uk_index_t in_offset,
+                    iree_uk_index_t in_stride0, iree_uk_index_t in_stride1,
+                    void* out_buffer, iree_uk_index_t out_offset,
+                    iree_uk_index_t out_stride0, iree_uk_index_t out_stride1,
+                    iree_uk_index_t in_size0, iree_uk_index_t in_size1,
+                    iree_uk_index_t in_size2, iree_uk_index_t in_size3,
+                    iree_uk_index_t out_size0, iree_uk_index_t out_size1,
+                    uint32_t flags, const uint64_t* cpu_data);
+void iree_uk_unpack_p(const iree_uk_unpack_params_t* params);
+
+/* Tile sizes the matmul kernels of this library prefer for an operand.
+ * Replaces: query_tile_sizes.h:29-31, query_tile_sizes.c:34-75. */
+void iree_uk_query_tile_sizes_2d(
+    const iree_uk_query_tile_sizes_2d_params_t* params,
+    iree_uk_query_tile_sizes_2d_out_params_t* out_params);
+
+/* Called when a parameter check or a HIP call fails. The library provides a
+ * weak default that prints to stderr and aborts; an embedder may define its
+ * own (reference: common.h:307-321 leaves the definition to the embedder). If
+ * the handler returns, the entry point returns without launching anything. */
+void iree_uk_assert_fail(const char* file, int line, const char* function,
+                         const char* condition);
+
+/*===--------------------------------------------------------------------===*/
+/* Entry points without a counterpart in the reference.                       */
+/*===--------------------------------------------------------------------===*/
+
+/* Library version, MAJOR*10000 + MINOR*100 + PATCH. */
+int iree_uk_mi355x_version(void);
+
+/* Selects the HIP device for the calling thread's launches and checks that it
+ * is a gfx950 part. Returns 0 on success, a HIP error code otherwise. Calling
+ * it is optional: the first launch uses the current HIP device. */
+int iree_uk_mi355x_init(int device_ordinal);
+
+/* Per-thread launch mode.
+ *   stream:  a hipStream_t cast to void* (NULL = the HIP null stream).
+ *   asynchronous == 0 (default): each entry point returns after its results are
+ *     visible, like the CPU microkernels. Operands whose `buffer + offset` is
+ *     not a device address are staged: copied to device memory owned by the
+ *     library, computed there, and the touched rows copied back.
+ *   asynchronous != 0: entry points only enqueue work on `stream` and return;
+ *     every operand must be device-accessible; nothing is staged or
+ *     synchronised. */
+void iree_uk_mi355x_set_stream(void* stream, int asynchronous);
+
+/* Replaces the failure handler for the calling process (NULL restores
+ * iree_uk_assert_fail). Meant for hosts that cannot provide a strong
+ * iree_uk_assert_fail symbol at link time. */
+typedef void (*iree_uk_mi355x_fail_handler_t)(const char* file, int line,
+                                              const char* function,
+                                              const char* condition);
+void iree_uk_mi355x_set_fail_handler(iree_uk_mi355x_fail_handler_t handler);
+
+/* Name of the kernel the calling thread's most recent entry point launched
+ * ("" if it returned early). Static storage; do not free. */
+const char* iree_uk_mi355x_last_kernel(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* IREE_UK_MI355X_H_ */
