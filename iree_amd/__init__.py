@@ -1,0 +1,2 @@
+"""MI355X-native data-tiled matmul microkernels (mmt4d / pack / unpack)."""
+from . import abi  # noqa: F401
