@@ -1,8 +1,5 @@
-// Placeholder selectors until the specialised kernels land.
+// Placeholder selector until the skinny-matrix kernel lands.
 #include "uk_internal.h"
 namespace uk {
-Mmt4dLauncher select_mmt4d_i8_mfma(const Mmt4dArgs&, bool) { return nullptr; }
-Mmt4dLauncher select_mmt4d_f16_mfma(const Mmt4dArgs&, bool) { return nullptr; }
 Mmt4dLauncher select_mmt4d_gemv(const Mmt4dArgs&, bool) { return nullptr; }
-Mmt4dLauncher select_mmt4d_s8s4_mfma(const Mmt4dArgs&, bool) { return nullptr; }
 }  // namespace uk
