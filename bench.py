@@ -1,0 +1,317 @@
+"""Benchmark of the data-tiled matmul microkernels on one MI355X.
+
+Headline workload (one "step" = one launch): iree_uk_mmt4d, s8s8s32, logical
+4096x4096x4096 with the 8x8x4 tiles of the reference's int8 configuration
+(lhs [512,1024,8,4], rhs [512,1024,8,4], out [512,512,8,8] int32), inputs
+resident in HBM. Prints ONE JSON line; besides the headline it carries the
+MFMA roofline of that kernel, the reference CPU ukernels timed on this host,
+and one-launch figures for the other configurations (pack/unpack GB/s, f16,
+skinny bf16, int4) under "also".
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-also]
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# Published MI355X peaks used for the roofline fractions.
+PEAK_INT8_TOPS = 5033.0     # dense int8 MFMA
+PEAK_F16_TFLOPS = 2516.0    # dense f16 / bf16 MFMA
+PEAK_HBM_GBS = 8000.0       # HBM3E
+
+
+def _mmt4d_params(abi, lhs, rhs, out, M, N, K, M0, N0, K0, flags):
+    lb, rb, ob = abi.MMT4D_BITS[flags & 0xFF]
+    p = abi.Mmt4dParams()
+    p.lhs_buffer, p.rhs_buffer, p.out_buffer = lhs, rhs, out
+    p.lhs_stride0, p.rhs_stride0, p.out_stride0 = K * M0 * K0, K * N0 * K0, N * M0 * N0
+    p.M, p.N, p.K, p.M0, p.N0, p.K0, p.flags = M, N, K, M0, N0, K0, flags
+    return p
+
+
+def _time_launches(torch, fn, steps, warmup):
+    """Average ms per call of fn() over `steps` calls, by HIP events on the
+    stream the kernels are launched on, bracketed by device synchronisation."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return e0.elapsed_time(e1) / steps, wall_ms / steps
+
+
+def _headline(torch, lib, abi, synth, steps, warmup):
+    import numpy as np
+    M = N = 512
+    K = 1024
+    M0 = N0 = 8
+    K0 = 4
+    flags = abi.MMT4D_TYPE_S8S8S32
+    lhs = torch.from_numpy(synth.uniform_int8(0, 0, M * K * M0 * K0)).cuda()
+    rhs = torch.from_numpy(synth.uniform_int8(0, 1, N * K * N0 * K0)).cuda()
+    out = torch.empty(M * N * M0 * N0, dtype=torch.int32, device="cuda")
+    p = _mmt4d_params(abi, lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), M, N, K, M0, N0, K0, flags)
+    ev_ms, wall_ms = _time_launches(torch, lambda: lib.iree_uk_mmt4d_p(C.byref(p)), steps, warmup)
+    kernel = lib.iree_uk_mi355x_last_kernel().decode()
+    # Checksum of checksums, independent of any CPU code: the sum of all
+    # outputs equals (column sums of A) . (column sums of B), with k running
+    # over (k, k0) pairs.
+    a_cols = lhs.view(M, K, M0, K0).to(torch.int64).sum(dim=(0, 2)).reshape(-1)
+    b_cols = rhs.view(N, K, N0, K0).to(torch.int64).sum(dim=(0, 2)).reshape(-1)
+    verified = bool((a_cols * b_cols).sum().item() == out.to(torch.int64).sum().item())
+    ops = 2.0 * M * N * K * M0 * N0 * K0
+    return dict(ops=ops, ev_ms=ev_ms, wall_ms=wall_ms, kernel=kernel, verified=verified,
+                workload="iree_uk_mmt4d s8s8s32 logical 4096x4096x4096, tiles M0=N0=8 K0=4 "
+                         "(lhs [512,1024,8,4], rhs [512,1024,8,4], out i32 [512,512,8,8]), "
+                         "accumulate off, operands resident in HBM")
+
+
+def _also(torch, lib, abi, synth, steps, warmup):
+    """One-launch figures for the other configurations."""
+    import numpy as np
+    res = {}
+
+    def mm(name, flags, M, N, K, M0, N0, K0, lhs, rhs, out_dtype, peak, unit, acc=False, bytes_model=None):
+        out = torch.zeros(M * N * M0 * N0, dtype=out_dtype, device="cuda")
+        p = _mmt4d_params(abi, lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), M, N, K, M0, N0, K0,
+                          flags | (abi.MMT4D_ACCUMULATE if acc else 0))
+        ms, _ = _time_launches(torch, lambda: lib.iree_uk_mmt4d_p(C.byref(p)), steps, warmup)
+        ops = 2.0 * M * N * K * M0 * N0 * K0
+        entry = {"kernel": lib.iree_uk_mi355x_last_kernel().decode(), "ms": round(ms, 5)}
+        if bytes_model is None:
+            entry.update({"value": round(ops / ms / 1e9, 1), "unit": unit,
+                          "frac_of_peak": round(ops / ms / 1e9 / peak, 4)})
+        else:
+            entry.update({"value": round(bytes_model / ms / 1e6, 1), "unit": "GB/s",
+                          "frac_of_peak": round(bytes_model / ms / 1e6 / PEAK_HBM_GBS, 4),
+                          "gflops": round(ops / ms / 1e6, 1)})
+        res[name] = entry
+
+    def f16_operand(seed, stream, n, sigma, bf16=False):
+        x = synth.normal_f32(seed, stream, n, sigma)
+        bits = synth.bf16_bits(x) if bf16 else synth.f16_bits(x)
+        return torch.from_numpy(bits.view(np.int16)).cuda()
+
+    # f16f16f32 4096^3, tiles 16x16x16, accumulate on.
+    n = 4096 * 4096
+    mm("mmt4d_f16f16f32_4096_16x16x16_acc", abi.MMT4D_TYPE_F16F16F32, 256, 256, 256, 16, 16, 16,
+       f16_operand(3, 0, n, 1.0 / 64), f16_operand(3, 1, n, 1.0 / 64), torch.float32,
+       PEAK_F16_TFLOPS, "TFLOP/s", acc=True)
+    # s8s4s32 512 x 11008 x 4096, tiles 16x16x32.
+    lhs = torch.from_numpy(synth.uniform_int8(5, 0, 512 * 4096)).cuda()
+    rhs = torch.from_numpy(synth.uniform_int4_packed(5, 1, 11008 * 4096).view(np.int8)).cuda()
+    mm("mmt4d_s8s4s32_512x11008x4096_16x16x32", abi.MMT4D_TYPE_S8S4S32, 32, 688, 128, 16, 16, 32,
+       lhs, rhs, torch.int32, PEAK_INT8_TOPS, "TOP/s")
+    # bf16 skinny shapes: M0 in {1, 4, 16}, N = 14336, K = 4096; HBM-bound on the
+    # rhs. Three rhs copies are rotated so the 256 MB last-level cache cannot
+    # serve them.
+    nk = 14336 * 4096
+    rhs_set = [f16_operand(4, 10 + i, nk, 0.02, bf16=True) for i in range(3)]
+    for m0 in (1, 4, 16):
+        lhs = f16_operand(4, m0, m0 * 4096, 1.0, bf16=True)
+        outs = torch.zeros(896 * m0 * 16, dtype=torch.float32, device="cuda")
+        ps = [_mmt4d_params(abi, lhs.data_ptr(), r.data_ptr(), outs.data_ptr(), 1, 896, 512, m0, 16, 8,
+                            abi.MMT4D_TYPE_BF16BF16F32) for r in rhs_set]
+        state = {"i": 0}
+
+        def step():
+            lib.iree_uk_mmt4d_p(C.byref(ps[state["i"] % 3]))
+            state["i"] += 1
+        ms, _ = _time_launches(torch, step, max(steps, 6), warmup)
+        nbytes = nk * 2 + m0 * 4096 * 2 + 896 * 16 * m0 * 4
+        res["mmt4d_bf16_skinny_M%d_N14336_K4096" % m0] = {
+            "kernel": lib.iree_uk_mi355x_last_kernel().decode(), "ms": round(ms, 5),
+            "value": round(nbytes / ms / 1e6, 1), "unit": "GB/s",
+            "frac_of_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+    del rhs_set
+
+    # pack / unpack f32 [8191, 8190] <-> [512, 8190, 16, 1]; two buffer sets rotated
+    # (each set is 537 MB, beyond the last-level cache).
+    R, Cc = 8191, 8190
+    src = [torch.from_numpy(synth.normal_f32(2, i, R * Cc)).cuda() for i in range(2)]
+    packed = [torch.empty(512 * Cc * 16, dtype=torch.float32, device="cuda") for _ in range(2)]
+    back = [torch.empty(R * Cc, dtype=torch.float32, device="cuda") for _ in range(2)]
+
+    def pack_params(i, flags, o0, o1, t0, t1):
+        p = abi.PackParams()
+        p.in_buffer, p.out_buffer = src[i].data_ptr(), packed[i].data_ptr()
+        p.in_stride0, p.in_stride1 = Cc, 1
+        p.out_stride0, p.out_stride1 = o1 * t0 * t1, t0 * t1
+        p.in_size0, p.in_size1 = R, Cc
+        p.out_size0, p.out_size1, p.out_size2, p.out_size3 = o0, o1, t0, t1
+        p.padding_value = 0
+        p.flags = abi.PACK_TYPE_F32F32 | flags
+        return p
+
+    def timed_pair(name, make, nbytes):
+        ps = [make(0), make(1)]
+        state = {"i": 0}
+
+        def step():
+            fn, p = ps[state["i"] & 1]
+            fn(C.byref(p))
+            state["i"] += 1
+        ms, _ = _time_launches(torch, step, max(steps, 6), warmup)
+        res[name] = {"kernel": lib.iree_uk_mi355x_last_kernel().decode(), "ms": round(ms, 5),
+                     "value": round(nbytes / ms / 1e6, 1), "unit": "GB/s",
+                     "frac_of_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+
+    timed_pair("pack_f32_8191x8190_to_512x8190x16x1",
+               lambda i: (lib.iree_uk_pack_p, pack_params(i, 0, 512, Cc, 16, 1)),
+               (R * Cc + 512 * Cc * 16) * 4)
+    # "Transposed-inner" variant: same out sizes (.., 16, 1) with TRANSPOSE_INNER,
+    # i.e. 1x16 tiles along dim 1: out [8191, 512, 16, 1].
+    packed2 = [torch.empty(R * 512 * 16, dtype=torch.float32, device="cuda") for _ in range(2)]
+
+    def pack_tr(i):
+        p = pack_params(i, abi.PACK_TRANSPOSE_INNER, R, 512, 16, 1)
+        p.out_buffer = packed2[i].data_ptr()
+        return (lib.iree_uk_pack_p, p)
+    timed_pair("pack_f32_8191x8190_transpose_inner_to_8191x512x16x1", pack_tr,
+               (R * Cc + R * 512 * 16) * 4)
+    del packed2
+
+    def unpack_params(i):
+        p = abi.UnpackParams()
+        p.in_buffer, p.out_buffer = packed[i].data_ptr(), back[i].data_ptr()
+        p.in_stride0, p.in_stride1 = Cc * 16, 16
+        p.out_stride0, p.out_stride1 = Cc, 1
+        p.in_size0, p.in_size1, p.in_size2, p.in_size3 = 512, Cc, 16, 1
+        p.out_size0, p.out_size1 = R, Cc
+        p.flags = abi.UNPACK_TYPE_F32F32
+        return (lib.iree_uk_unpack_p, p)
+    # Make sure `packed` holds packed data for both sets, then time unpack.
+    for i in range(2):
+        lib.iree_uk_pack_p(C.byref(pack_params(i, 0, 512, Cc, 16, 1)))
+    timed_pair("unpack_f32_512x8190x16x1_to_8191x8190", unpack_params, 2 * R * Cc * 4)
+    torch.cuda.synchronize()
+    res["pack_unpack_round_trip_bit_exact"] = bool(all(torch.equal(src[i], back[i]) for i in range(2)))
+    return res
+
+
+def _cpu_baseline(abi, synth, threads):
+    """The reference CPU ukernels (compiled from the reference's own sources into
+    oracle/_ref) on this host; falls back to this repository's scalar port."""
+    import numpy as np
+    import oracle
+    ref = oracle.ref_lib()
+    # Bounded sample of the headline workload: the first 64 of its 512 rows of
+    # 8x8 tiles against all 512 rhs panels, full K (1/8 of the work).
+    Ms, N, K, M0, N0, K0 = 64, 512, 1024, 8, 8, 4
+    lhs = synth.uniform_int8(0, 0, 512 * K * M0 * K0)[:Ms * K * M0 * K0]
+    rhs = synth.uniform_int8(0, 1, N * K * N0 * K0)
+    out = np.zeros(Ms * N * M0 * N0, dtype=np.int32)
+    cpu = oracle.host_cpu_data()
+    p = _mmt4d_params(abi, lhs.ctypes.data, rhs.ctypes.data, out.ctypes.data, Ms, N, K, M0, N0, K0,
+                      abi.MMT4D_TYPE_S8S8S32 | abi.MMT4D_ALLOW_GENERIC_FALLBACK)
+    p.cpu_data = C.cast(cpu, C.POINTER(C.c_uint64))
+    if ref is not None:
+        run, kind = (lambda: ref.ref_mmt4d_mt(C.byref(p), threads)), "reference"
+    else:
+        run, kind = (lambda: oracle.lib().oracle_mmt4d_mt(C.byref(p), threads)), "port"
+    best = None
+    for _ in range(2):
+        t0 = time.perf_counter()
+        run()
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    ops = 2.0 * Ms * N * K * M0 * N0 * K0
+    base = {"value": round(ops / best / 1e12, 5), "unit": "TOP/s", "cores": threads, "kind": kind,
+            "sample": "rows 0..63 of the 512 rows of 8x8 lhs tiles x all 512 rhs panels x full K "
+                      "(1/8 of the headline workload), generic tile function (the reference has no "
+                      "x86-64 tile for 8x8x4), best of 2"}
+    extra = None
+    if ref is not None:
+        # The reference's architecture-specific tiles need its own tile shape:
+        # s8s8s32 16x16x2 (AVX-512 VNNI where the host has it), same logical size.
+        M, N, K, M0, N0, K0 = 256, 256, 2048, 16, 16, 2
+        lhs = synth.uniform_int8(0, 0, M * K * M0 * K0)
+        rhs = synth.uniform_int8(0, 1, N * K * N0 * K0)
+        out = np.zeros(M * N * M0 * N0, dtype=np.int32)
+        q = _mmt4d_params(abi, lhs.ctypes.data, rhs.ctypes.data, out.ctypes.data, M, N, K, M0, N0, K0,
+                          abi.MMT4D_TYPE_S8S8S32 | abi.MMT4D_ALLOW_GENERIC_FALLBACK)
+        q.cpu_data = C.cast(cpu, C.POINTER(C.c_uint64))
+        has_arch = bool(ref.ref_mmt4d_info(C.byref(q)) & 1)
+        best = None
+        for _ in range(2):
+            t0 = time.perf_counter()
+            ref.ref_mmt4d_mt(C.byref(q), threads)
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        extra = {"value": round(2.0 * 4096 ** 3 / best / 1e12, 5), "unit": "TOP/s", "cores": threads,
+                 "kind": "reference",
+                 "sample": "full 4096^3 in the reference's own x86-64 tile shape 16x16x2, "
+                           "architecture-specific tile function %s, best of 2"
+                           % ("selected" if has_arch else "NOT available on this host (generic used)")}
+    return base, extra
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-also", action="store_true", help="headline workload only")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this library runs on ONE GPU (a ukernel call has no cross-device "
+                 "part); --gpus %d is not supported, use --gpus 1" % args.gpus)
+
+    import torch
+    from iree_amd import abi, library, synth
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    lib = library.load()  # raises if the HIP library is missing: no fallback
+    rc = lib.iree_uk_mi355x_init(0)
+    if rc != 0:
+        sys.exit("bench.py: device 0 is not usable as a gfx950 part (code %d)" % rc)
+    torch.cuda.set_device(0)
+    lib.iree_uk_mi355x_set_stream(torch.cuda.current_stream().cuda_stream, 1)
+
+    head = _headline(torch, lib, abi, synth, args.steps, args.warmup)
+    also = None if args.no_also else _also(torch, lib, abi, synth, max(6, args.steps // 5), 2)
+    lib.iree_uk_mi355x_set_stream(None, 0)
+
+    threads = min(16, os.cpu_count() or 1)
+    cpu, cpu_arch = (None, None) if args.no_cpu else _cpu_baseline(abi, synth, threads)
+
+    tops = head["ops"] / head["ev_ms"] / 1e9
+    line = {
+        "metric": "mmt4d s8s8s32 throughput at logical 4096^3 on 1 MI355X",
+        "value": round(head["ops"] / head["wall_ms"] / 1e9, 2),
+        "unit": "TOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(head["wall_ms"], 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8", "data": "synthetic",
+        "config": {"workload": head["workload"], "kernel": head["kernel"],
+                   "checksum_verified": head["verified"]},
+        "roofline": {"bound": "mfma", "achieved": round(tops, 2), "peak": PEAK_INT8_TOPS,
+                     "unit": "TOP/s", "frac": round(tops / PEAK_INT8_TOPS, 4), "traffic": None,
+                     "kernel_ms": round(head["ev_ms"], 5)},
+        "cpu_baseline": cpu,
+    }
+    if cpu_arch is not None:
+        line["cpu_baseline_arch_tiles"] = cpu_arch
+    if also is not None:
+        line["also"] = also
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
