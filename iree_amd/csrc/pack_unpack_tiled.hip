@@ -1,4 +1,23 @@
-// Selection between the LDS-staged pack/unpack kernels and the generic ones.
+// LDS-staged pack / unpack for power-of-two tile sizes: HBM-bandwidth kernels.
+//
+// A workgroup owns a BR x BC block of the 2-D matrix (BR a multiple of the tile
+// height T0, BC a multiple of the tile width T1). The block's image in the
+// tiled buffer is a small number of long contiguous runs: with no outer
+// transpose the BC/T1 tiles of one tile row follow each other, with an outer
+// transpose the BR/T0 tiles of one tile column do. So both sides of the copy
+// can be done with wide, fully coalesced accesses and the re-ordering happens
+// in LDS:
+//   pack:    2-D rows -> LDS (row-major, padded pitch) -> tiled runs (128-bit)
+//   unpack:  tiled runs (128-bit) -> LDS -> 2-D rows
+// The 2-D side uses the widest vector (16, 8 or 4 bytes, else one element)
+// that the row alignment allows. Element values are never interpreted: the
+// kernels move bytes, so results are bit-exact by construction; padding is the
+// low bytes of padding_value (pack.h:15-24).
+//
+// Anything this file does not cover (non power-of-two tiles, inner stride on
+// the 2-D side, unaligned tiled buffers) goes to the generic kernels.
+#include <type_traits>
+
 #include "uk_internal.h"
 
 namespace uk {
@@ -6,12 +25,395 @@ namespace uk {
 hipError_t launch_pack_generic(const PackArgs& a, hipStream_t stream, const char** name);
 hipError_t launch_unpack_generic(const UnpackArgs& a, hipStream_t stream, const char** name);
 
+namespace {
+
+struct TiledArgs {
+  const uint8_t* src;   // pack: 2-D buffer, unpack: tiled buffer
+  uint8_t* dst;         // pack: tiled buffer, unpack: 2-D buffer
+  int64_t flat_stride0;   // 2-D side row stride, elements
+  int64_t tiled_stride0;  // tiled side outer stride, elements
+  int64_t size0, size1;   // 2-D sizes
+  int64_t outer0, outer1; // tile counts along 2-D dims 0 / 1
+  uint64_t padding_value;
+  int32_t log2_t0, log2_t1;  // tile sizes along 2-D dims 0 / 1
+  int32_t log2_s3;           // log2 of the tiled buffer's innermost size
+  int32_t log2_br, log2_bc;  // block shape
+  int32_t pitch_bytes;       // LDS row pitch
+  int32_t blocks1;           // blocks along dim 1
+  int32_t tr_inner, tr_outer;
+};
+
+// Coordinates of an element of the tiled side within a block.
+struct TiledCoord {
+  int64_t global_elem;  // element offset in the tiled buffer
+  int32_t row, col;     // position in the block (2-D side)
+  bool in_range;        // tile exists in the tiled buffer
+};
+
+// Element `e` (in the block's tiled-side enumeration: runs in order, each run
+// tile after tile, each tile in stored order) -> where it lives.
+__device__ __forceinline__ TiledCoord tiled_coord(const TiledArgs& a, int32_t e, int64_t tile0_base,
+                                                  int64_t tile1_base) {
+  const int32_t log2_tile = a.log2_t0 + a.log2_t1;
+  int32_t o0l, o1l, w;
+  if (!a.tr_outer) {
+    const int32_t log2_run = a.log2_bc + a.log2_t0;  // elements per run (one tile row of the block)
+    o0l = e >> log2_run;
+    const int32_t rem = e & ((1 << log2_run) - 1);
+    o1l = rem >> log2_tile;
+    w = rem & ((1 << log2_tile) - 1);
+  } else {
+    const int32_t log2_run = a.log2_br + a.log2_t1;  // one tile column of the block
+    o1l = e >> log2_run;
+    const int32_t rem = e & ((1 << log2_run) - 1);
+    o0l = rem >> log2_tile;
+    w = rem & ((1 << log2_tile) - 1);
+  }
+  const int32_t u2 = w >> a.log2_s3, u3 = w & ((1 << a.log2_s3) - 1);
+  const int32_t t0 = a.tr_inner ? u3 : u2, t1 = a.tr_inner ? u2 : u3;
+  TiledCoord c;
+  c.row = (o0l << a.log2_t0) + t0;
+  c.col = (o1l << a.log2_t1) + t1;
+  const int64_t o0 = tile0_base + o0l, o1 = tile1_base + o1l;
+  c.in_range = o0 < a.outer0 && o1 < a.outer1;
+  const int64_t q0 = a.tr_outer ? o1 : o0, q1 = a.tr_outer ? o0 : o1;
+  c.global_elem = q0 * a.tiled_stride0 + (q1 << log2_tile) + w;
+  return c;
+}
+
+template <typename T>
+__device__ __forceinline__ T pad_value(uint64_t v) { return (T)v; }
+
+// E: element bytes. W: vector bytes on the 2-D side. PL_BYTES: bytes of one
+// contiguous LDS piece on the tiled side (16 when 16 output bytes come from one
+// LDS row, down to E for column access).
+template <int E, int W, int PL_BYTES, bool UNPACK>
+__global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  typedef typename std::conditional<E == 1, uint8_t,
+          typename std::conditional<E == 2, uint16_t, uint32_t>::type>::type elem_t;
+  typedef typename std::conditional<W == 16, uint4,
+          typename std::conditional<W == 8, uint2,
+          typename std::conditional<W == 4, uint32_t,
+          typename std::conditional<W == 2, uint16_t, uint8_t>::type>::type>::type>::type flat_vec_t;
+  static_assert(sizeof(flat_vec_t) == W && W >= E, "2-D side vector type");
+  typedef typename std::conditional<PL_BYTES == 16, uint4,
+          typename std::conditional<PL_BYTES == 8, uint2,
+          typename std::conditional<PL_BYTES == 4, uint32_t,
+          typename std::conditional<PL_BYTES == 2, uint16_t, uint8_t>::type>::type>::type>::type piece_t;
+  constexpr int VE = 16 / E;          // elements per 128-bit tiled-side vector
+  constexpr int PIECES = 16 / PL_BYTES;
+  constexpr int PL = PL_BYTES / E;    // elements per piece
+
+  const int tid = threadIdx.x;
+  const int64_t block0 = blockIdx.x / a.blocks1, block1 = blockIdx.x % a.blocks1;
+  const int64_t row_base = block0 << a.log2_br, col_base = block1 << a.log2_bc;
+  const int64_t tile0_base = row_base >> a.log2_t0, tile1_base = col_base >> a.log2_t1;
+  const int32_t BR = 1 << a.log2_br, BC = 1 << a.log2_bc;
+  const int32_t block_elems = BR * BC;
+
+  // ---- 2-D side <-> LDS ----
+  auto flat_phase = [&]() {
+    const int32_t vec_per_row = (BC * E) / W;
+    const int32_t log2_vpr = a.log2_bc + (E == 1 ? 0 : E == 2 ? 1 : 2) - (W == 16 ? 4 : W == 8 ? 3 : W == 4 ? 2 : W == 2 ? 1 : 0);
+    const int32_t total = BR * vec_per_row;
+    constexpr int EPV = W / E;  // elements per 2-D side vector
+    for (int32_t v = tid; v < total; v += 256) {
+      const int32_t r = v >> log2_vpr, cv = v & (vec_per_row - 1);
+      const int64_t row = row_base + r, col = col_base + (int64_t)cv * EPV;
+      uint8_t* l = lds + r * a.pitch_bytes + cv * W;
+      if constexpr (!UNPACK) {
+        const uint8_t* g = a.src + (row * a.flat_stride0 + col) * E;
+        if (row < a.size0 && col + EPV <= a.size1) {
+          *(flat_vec_t*)l = *(const flat_vec_t*)g;
+        } else {
+          // Edge: element by element, padding where the input ends.
+#pragma unroll
+          for (int i = 0; i < EPV; ++i) {
+            elem_t x = pad_value<elem_t>(a.padding_value);
+            if (row < a.size0 && col + i < a.size1) x = ((const elem_t*)g)[i];
+            ((elem_t*)l)[i] = x;
+          }
+        }
+      } else {
+        uint8_t* g = a.dst + (row * a.flat_stride0 + col) * E;
+        if (row < a.size0 && col + EPV <= a.size1) {
+          *(flat_vec_t*)g = *(const flat_vec_t*)l;
+        } else if (row < a.size0) {
+#pragma unroll
+          for (int i = 0; i < EPV; ++i)
+            if (col + i < a.size1) ((elem_t*)g)[i] = ((const elem_t*)l)[i];
+        }
+      }
+    }
+  };
+
+  // ---- tiled side <-> LDS ----
+  auto tiled_phase = [&]() {
+    const int32_t total = block_elems / VE;
+    for (int32_t v = tid; v < total; v += 256) {
+      const int32_t e = v * VE;
+      const TiledCoord c0 = tiled_coord(a, e, tile0_base, tile1_base);
+      if (!c0.in_range) continue;
+      union { uint4 vec; piece_t piece[PIECES]; } u;
+      if constexpr (!UNPACK) {
+        if constexpr (PIECES == 1) {
+          u.vec = *(const uint4*)(lds + c0.row * a.pitch_bytes + c0.col * E);
+        } else {
+#pragma unroll
+          for (int q = 0; q < PIECES; ++q) {
+            const TiledCoord c = tiled_coord(a, e + q * PL, tile0_base, tile1_base);
+            u.piece[q] = *(const piece_t*)(lds + c.row * a.pitch_bytes + c.col * E);
+          }
+        }
+        *(uint4*)(a.dst + c0.global_elem * E) = u.vec;
+      } else {
+        u.vec = *(const uint4*)(a.src + c0.global_elem * E);
+        if constexpr (PIECES == 1) {
+          *(uint4*)(lds + c0.row * a.pitch_bytes + c0.col * E) = u.vec;
+        } else {
+#pragma unroll
+          for (int q = 0; q < PIECES; ++q) {
+            const TiledCoord c = tiled_coord(a, e + q * PL, tile0_base, tile1_base);
+            *(piece_t*)(lds + c.row * a.pitch_bytes + c.col * E) = u.piece[q];
+          }
+        }
+      }
+    }
+  };
+
+  if constexpr (!UNPACK) {
+    flat_phase();
+    __syncthreads();
+    tiled_phase();
+  } else {
+    tiled_phase();
+    __syncthreads();
+    flat_phase();
+  }
+}
+
+int log2_exact(int64_t v) {
+  if (v <= 0 || (v & (v - 1))) return -1;
+  int l = 0;
+  while ((1ll << l) < v) ++l;
+  return l;
+}
+
+int largest_pow2_dividing(uint64_t v, int cap) {
+  int w = 1;
+  while (w < cap && (v % (2 * w)) == 0) w *= 2;
+  return w;
+}
+
+// Host copy of tiled_coord's (row, col) for the bank-conflict search below.
+void host_row_col(const TiledArgs& a, int32_t e, int32_t* row, int32_t* col) {
+  const int32_t log2_tile = a.log2_t0 + a.log2_t1;
+  int32_t o0l, o1l, w;
+  if (!a.tr_outer) {
+    const int32_t log2_run = a.log2_bc + a.log2_t0;
+    o0l = e >> log2_run;
+    const int32_t rem = e & ((1 << log2_run) - 1);
+    o1l = rem >> log2_tile;
+    w = rem & ((1 << log2_tile) - 1);
+  } else {
+    const int32_t log2_run = a.log2_br + a.log2_t1;
+    o1l = e >> log2_run;
+    const int32_t rem = e & ((1 << log2_run) - 1);
+    o0l = rem >> log2_tile;
+    w = rem & ((1 << log2_tile) - 1);
+  }
+  const int32_t u2 = w >> a.log2_s3, u3 = w & ((1 << a.log2_s3) - 1);
+  const int32_t t0 = a.tr_inner ? u3 : u2, t1 = a.tr_inner ? u2 : u3;
+  *row = (o0l << a.log2_t0) + t0;
+  *col = (o1l << a.log2_t1) + t1;
+}
+
+// LDS row pitch: the block width plus the padding (in 16-byte steps) that
+// spreads one wavefront's tiled-side accesses over the most of the 64 banks.
+int choose_pitch(const TiledArgs& a, int elem_bytes, int piece_bytes) {
+  const int row_bytes = (1 << a.log2_bc) * elem_bytes;
+  const int ve = 16 / elem_bytes;
+  int best_pitch = row_bytes, best_cost = 1 << 30;
+  for (int pad = 0; pad <= 256; pad += 16) {
+    const int pitch = row_bytes + pad;
+    int hits[64] = {0};
+    for (int lane = 0; lane < 64; ++lane) {
+      int32_t row, col;
+      host_row_col(a, lane * ve, &row, &col);
+      const int addr = row * pitch + col * elem_bytes;
+      const int words = piece_bytes < 4 ? 1 : piece_bytes / 4;
+      for (int w = 0; w < words; ++w) hits[((addr / 4) + w) & 63]++;
+    }
+    int cost = 0;
+    for (int b = 0; b < 64; ++b) cost = hits[b] > cost ? hits[b] : cost;
+    if (cost < best_cost) {
+      best_cost = cost;
+      best_pitch = pitch;
+    }
+  }
+  return best_pitch;
+}
+
+struct Plan {
+  TiledArgs args;
+  int elem_bytes, flat_vec_bytes, piece_bytes;
+  unsigned grid;
+  size_t lds_bytes;
+};
+
+// Common planning for pack and unpack. `flat` is the 2-D side, `tiled` the
+// 4-D side; returns false if the generic kernel has to take the call.
+bool make_plan(const uint8_t* flat, const uint8_t* tiled, int64_t flat_stride0, int64_t flat_stride1,
+               int64_t tiled_stride0, int64_t size0, int64_t size1, int64_t tsize0, int64_t tsize1,
+               int64_t tsize2, int64_t tsize3, bool tr_inner, bool tr_outer, int elem_bytes,
+               Plan* plan) {
+  if (flat_stride1 != 1) return false;
+  const int l2 = log2_exact(tsize2), l3 = log2_exact(tsize3);
+  if (l2 < 0 || l3 < 0) return false;
+  const int64_t tile_bytes = tsize2 * tsize3 * elem_bytes;
+  if (tile_bytes % 16 || tile_bytes > 16384) return false;
+  if ((uintptr_t)tiled % 16 || (tiled_stride0 * elem_bytes) % 16) return false;
+  if ((uintptr_t)flat % elem_bytes) return false;
+  if (size0 <= 0 || size1 <= 0) return false;  // nothing but padding: generic
+
+  TiledArgs& a = plan->args;
+  a.tr_inner = tr_inner;
+  a.tr_outer = tr_outer;
+  a.log2_s3 = l3;
+  a.log2_t0 = tr_inner ? l3 : l2;
+  a.log2_t1 = tr_inner ? l2 : l3;
+  a.outer0 = tr_outer ? tsize1 : tsize0;
+  a.outer1 = tr_outer ? tsize0 : tsize1;
+  a.flat_stride0 = flat_stride0;
+  a.tiled_stride0 = tiled_stride0;
+  a.size0 = size0;
+  a.size1 = size1;
+  const int64_t T0 = 1ll << a.log2_t0, T1 = 1ll << a.log2_t1;
+
+  // Block shape: rows of at least 256 bytes on the 2-D side, runs of at least
+  // 1 KiB on the tiled side, about 16 KiB per block.
+  const int E = elem_bytes;
+  int64_t bc = 256 / E, br = T0;
+  if (bc < T1) bc = T1;
+  if (!tr_outer) {
+    while (bc * T0 * E < 1024) bc *= 2;
+  } else {
+    while (br * T1 * E < 1024) br *= 2;
+  }
+  while (br * bc * E < 16384) {
+    // Grow the dimension that lengthens the runs first, then the other.
+    if (!tr_outer) { if (bc * E < 2048) bc *= 2; else br *= 2; }
+    else { if (br * T1 * E < 4096) br *= 2; else bc *= 2; }
+  }
+  while (br * bc * E > 32768 && br > T0) br /= 2;
+  while (br * bc * E > 32768 && bc > T1 && bc * E > 256) bc /= 2;
+  if (br * bc * E > 49152) return false;
+  a.log2_br = log2_exact(br);
+  a.log2_bc = log2_exact(bc);
+
+  // Vector width on the 2-D side from the alignment shared by all rows.
+  int w = largest_pow2_dividing((uintptr_t)flat, 16);
+  if (size0 > 1) {
+    const int ws = largest_pow2_dividing((uint64_t)(flat_stride0 * E), 16);
+    w = ws < w ? ws : w;
+  }
+  if (w < E) w = E;
+  plan->flat_vec_bytes = w;
+
+  // Contiguous LDS piece on the tiled side.
+  int piece = tr_inner ? E : (int)((T1 * E) < 16 ? (T1 * E) : 16);
+  plan->piece_bytes = piece;
+  plan->elem_bytes = E;
+
+  a.pitch_bytes = choose_pitch(a, E, piece);
+  a.blocks1 = (int32_t)((size1 + bc - 1) / bc);
+  // Blocks must cover every tile of the tiled side, not only the 2-D extent
+  // (pack writes whole tiles of padding beyond it).
+  const int64_t rows_needed = a.outer0 << a.log2_t0, cols_needed = a.outer1 << a.log2_t1;
+  const int64_t blocks0 = (rows_needed + br - 1) / br;
+  a.blocks1 = (int32_t)((cols_needed + bc - 1) / bc);
+  if (blocks0 * a.blocks1 >= (1ll << 31)) return false;
+  plan->grid = (unsigned)(blocks0 * a.blocks1);
+  plan->lds_bytes = (size_t)br * a.pitch_bytes;
+  return plan->lds_bytes <= 65536;
+}
+
+template <int E, int W, bool UNPACK>
+hipError_t launch_pw(const Plan& p, hipStream_t stream) {
+  const dim3 grid(p.grid), block(256);
+  switch (p.piece_bytes) {
+#define UK_PIECE(PB)                                                                         \
+  case PB:                                                                                   \
+    if constexpr (PB >= E) {                                                                 \
+      hipLaunchKernelGGL((tiled_kernel<E, W, PB, UNPACK>), grid, block, p.lds_bytes, stream, \
+                         p.args);                                                            \
+      return hipGetLastError();                                                              \
+    }                                                                                        \
+    return hipErrorInvalidValue
+    UK_PIECE(16);
+    UK_PIECE(8);
+    UK_PIECE(4);
+    UK_PIECE(2);
+    UK_PIECE(1);
+#undef UK_PIECE
+    default:
+      return hipErrorInvalidValue;
+  }
+}
+
+template <int E, bool UNPACK>
+hipError_t launch_e(const Plan& p, hipStream_t stream) {
+  switch (p.flat_vec_bytes) {
+    case 16: return launch_pw<E, 16, UNPACK>(p, stream);
+    case 8: return launch_pw<E, 8, UNPACK>(p, stream);
+    case 4: return launch_pw<E, 4, UNPACK>(p, stream);
+    case 2: if constexpr (E <= 2) return launch_pw<E, 2, UNPACK>(p, stream); return hipErrorInvalidValue;
+    case 1: if constexpr (E == 1) return launch_pw<E, 1, UNPACK>(p, stream); return hipErrorInvalidValue;
+    default: return hipErrorInvalidValue;
+  }
+}
+
+template <bool UNPACK>
+hipError_t launch_plan(const Plan& p, hipStream_t stream) {
+  switch (p.elem_bytes) {
+    case 1: return launch_e<1, UNPACK>(p, stream);
+    case 2: return launch_e<2, UNPACK>(p, stream);
+    case 4: return launch_e<4, UNPACK>(p, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace
+
 hipError_t launch_pack(const PackArgs& a, hipStream_t stream, const char** name) {
-  return launch_pack_generic(a, stream, name);
+  Plan plan;
+  const bool tr_inner = a.flags & IREE_UK_FLAG_PACK_TRANSPOSE_INNER;
+  const bool tr_outer = a.flags & IREE_UK_FLAG_PACK_TRANSPOSE_OUTER;
+  if (!make_plan(a.in, a.out, a.in_stride0, a.in_stride1, a.out_stride0, a.in_size0, a.in_size1,
+                 a.out_size0, a.out_size1, a.out_size2, a.out_size3, tr_inner, tr_outer,
+                 a.elem_bytes, &plan))
+    return launch_pack_generic(a, stream, name);
+  plan.args.src = a.in;
+  plan.args.dst = a.out;
+  plan.args.padding_value = a.padding_value;
+  *name = "pack_tiled";
+  return launch_plan<false>(plan, stream);
 }
 
 hipError_t launch_unpack(const UnpackArgs& a, hipStream_t stream, const char** name) {
-  return launch_unpack_generic(a, stream, name);
+  Plan plan;
+  const bool tr_inner = a.flags & IREE_UK_FLAG_UNPACK_TRANSPOSE_INNER;
+  const bool tr_outer = a.flags & IREE_UK_FLAG_UNPACK_TRANSPOSE_OUTER;
+  if (!make_plan(a.out, a.in, a.out_stride0, a.out_stride1, a.in_stride0, a.out_size0, a.out_size1,
+                 a.in_size0, a.in_size1, a.in_size2, a.in_size3, tr_inner, tr_outer, a.elem_bytes,
+                 &plan))
+    return launch_unpack_generic(a, stream, name);
+  plan.args.src = a.in;
+  plan.args.dst = a.out;
+  plan.args.padding_value = 0;
+  *name = "unpack_tiled";
+  return launch_plan<true>(plan, stream);
 }
 
 }  // namespace uk
