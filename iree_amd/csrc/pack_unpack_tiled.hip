@@ -40,6 +40,7 @@ struct TiledArgs {
   int32_t log2_br, log2_bc;  // block shape
   int32_t pitch_bytes;       // LDS row pitch
   int32_t blocks1;           // blocks along dim 1
+  int32_t total_blocks;
   int32_t tr_inner, tr_outer;
 };
 
@@ -81,115 +82,162 @@ __device__ __forceinline__ TiledCoord tiled_coord(const TiledArgs& a, int32_t e,
   return c;
 }
 
-template <typename T>
-__device__ __forceinline__ T pad_value(uint64_t v) { return (T)v; }
+// 16 bytes that only need 4-byte alignment: the hardware's multi-dword global
+// accesses do not require more, the C++ type system would.
+struct __attribute__((packed, aligned(4))) Dwords4 {
+  uint32_t x, y, z, w;
+};
 
-// E: element bytes. W: vector bytes on the 2-D side. PL_BYTES: bytes of one
-// contiguous LDS piece on the tiled side (16 when 16 output bytes come from one
-// LDS row, down to E for column access).
+constexpr int kBlockBytes = 16384;  // bytes of the 2-D matrix per workgroup
+
+// E: element bytes. W: vector bytes on the 2-D side (16 needs 4-byte aligned
+// rows). PL_BYTES: bytes of one contiguous LDS piece on the tiled side (16 when
+// 16 output bytes come from one LDS row, down to E for column access).
 template <int E, int W, int PL_BYTES, bool UNPACK>
 __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   typedef typename std::conditional<E == 1, uint8_t,
           typename std::conditional<E == 2, uint16_t, uint32_t>::type>::type elem_t;
-  typedef typename std::conditional<W == 16, uint4,
+  typedef typename std::conditional<W == 16, Dwords4,
           typename std::conditional<W == 8, uint2,
           typename std::conditional<W == 4, uint32_t,
           typename std::conditional<W == 2, uint16_t, uint8_t>::type>::type>::type>::type flat_vec_t;
-  static_assert(sizeof(flat_vec_t) == W && W >= E, "2-D side vector type");
   typedef typename std::conditional<PL_BYTES == 16, uint4,
           typename std::conditional<PL_BYTES == 8, uint2,
           typename std::conditional<PL_BYTES == 4, uint32_t,
           typename std::conditional<PL_BYTES == 2, uint16_t, uint8_t>::type>::type>::type>::type piece_t;
+  static_assert(sizeof(flat_vec_t) == W && W >= E, "2-D side vector type");
   constexpr int VE = 16 / E;          // elements per 128-bit tiled-side vector
   constexpr int PIECES = 16 / PL_BYTES;
   constexpr int PL = PL_BYTES / E;    // elements per piece
+  constexpr int EPV = W / E;          // elements per 2-D side vector
+  constexpr int FLAT_PER_THREAD = kBlockBytes / W / 256;
+  constexpr int TILED_PER_THREAD = kBlockBytes / 16 / 256;
+  constexpr int LOG2_E = E == 1 ? 0 : E == 2 ? 1 : 2;
+  constexpr int LOG2_W = W == 16 ? 4 : W == 8 ? 3 : W == 4 ? 2 : W == 2 ? 1 : 0;
 
   const int tid = threadIdx.x;
-  const int64_t block0 = blockIdx.x / a.blocks1, block1 = blockIdx.x % a.blocks1;
+  // Consecutive workgroup ids land on different XCDs (separate L2s). Regroup
+  // them so that one XCD owns a contiguous range of blocks: neighbours along a
+  // row share the cache lines at their common edge (rows need not be aligned
+  // to lines), and those then meet in one L2 instead of two.
+  const int32_t per_xcd = (a.total_blocks + 7) >> 3;
+  const int32_t linear = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (linear >= a.total_blocks) return;
+  const int64_t block0 = linear / a.blocks1, block1 = linear % a.blocks1;
   const int64_t row_base = block0 << a.log2_br, col_base = block1 << a.log2_bc;
   const int64_t tile0_base = row_base >> a.log2_t0, tile1_base = col_base >> a.log2_t1;
-  const int32_t BR = 1 << a.log2_br, BC = 1 << a.log2_bc;
-  const int32_t block_elems = BR * BC;
+  const int32_t log2_vpr = a.log2_bc + LOG2_E - LOG2_W;  // 2-D side vectors per block row
+  const int32_t vpr_mask = (1 << log2_vpr) - 1;
 
-  // ---- 2-D side <-> LDS ----
-  auto flat_phase = [&]() {
-    const int32_t vec_per_row = (BC * E) / W;
-    const int32_t log2_vpr = a.log2_bc + (E == 1 ? 0 : E == 2 ? 1 : 2) - (W == 16 ? 4 : W == 8 ? 3 : W == 4 ? 2 : W == 2 ? 1 : 0);
-    const int32_t total = BR * vec_per_row;
-    constexpr int EPV = W / E;  // elements per 2-D side vector
-    for (int32_t v = tid; v < total; v += 256) {
-      const int32_t r = v >> log2_vpr, cv = v & (vec_per_row - 1);
-      const int64_t row = row_base + r, col = col_base + (int64_t)cv * EPV;
-      uint8_t* l = lds + r * a.pitch_bytes + cv * W;
-      if constexpr (!UNPACK) {
+  union FlatVec {
+    flat_vec_t vec;
+    elem_t elem[EPV];
+  };
+
+  // ---- 2-D rows -> LDS (pack), all global loads issued before the LDS stores ----
+  auto flat_load_phase = [&]() {
+    constexpr int BATCH = FLAT_PER_THREAD < 8 ? FLAT_PER_THREAD : 8;
+    for (int u0 = 0; u0 < FLAT_PER_THREAD; u0 += BATCH) {
+      FlatVec regs[BATCH];
+#pragma unroll
+      for (int u = 0; u < BATCH; ++u) {
+        const int32_t v = tid + 256 * (u0 + u);
+        const int32_t r = v >> log2_vpr, cv = v & vpr_mask;
+        const int64_t row = row_base + r, col = col_base + (int64_t)cv * EPV;
         const uint8_t* g = a.src + (row * a.flat_stride0 + col) * E;
         if (row < a.size0 && col + EPV <= a.size1) {
-          *(flat_vec_t*)l = *(const flat_vec_t*)g;
+          regs[u].vec = *(const flat_vec_t*)g;
         } else {
           // Edge: element by element, padding where the input ends.
 #pragma unroll
           for (int i = 0; i < EPV; ++i) {
-            elem_t x = pad_value<elem_t>(a.padding_value);
+            elem_t x = (elem_t)a.padding_value;
             if (row < a.size0 && col + i < a.size1) x = ((const elem_t*)g)[i];
-            ((elem_t*)l)[i] = x;
+            regs[u].elem[i] = x;
           }
         }
-      } else {
+      }
+#pragma unroll
+      for (int u = 0; u < BATCH; ++u) {
+        const int32_t v = tid + 256 * (u0 + u);
+        const int32_t r = v >> log2_vpr, cv = v & vpr_mask;
+        *(flat_vec_t*)(lds + r * a.pitch_bytes + cv * W) = regs[u].vec;
+      }
+    }
+  };
+
+  // ---- LDS -> 2-D rows (unpack), nothing written outside size0 x size1 ----
+  auto flat_store_phase = [&]() {
+    constexpr int BATCH = FLAT_PER_THREAD < 8 ? FLAT_PER_THREAD : 8;
+    for (int u0 = 0; u0 < FLAT_PER_THREAD; u0 += BATCH) {
+      FlatVec regs[BATCH];
+#pragma unroll
+      for (int u = 0; u < BATCH; ++u) {
+        const int32_t v = tid + 256 * (u0 + u);
+        regs[u].vec = *(const flat_vec_t*)(lds + (v >> log2_vpr) * a.pitch_bytes + (v & vpr_mask) * W);
+      }
+#pragma unroll
+      for (int u = 0; u < BATCH; ++u) {
+        const int32_t v = tid + 256 * (u0 + u);
+        const int32_t r = v >> log2_vpr, cv = v & vpr_mask;
+        const int64_t row = row_base + r, col = col_base + (int64_t)cv * EPV;
         uint8_t* g = a.dst + (row * a.flat_stride0 + col) * E;
         if (row < a.size0 && col + EPV <= a.size1) {
-          *(flat_vec_t*)g = *(const flat_vec_t*)l;
+          *(flat_vec_t*)g = regs[u].vec;
         } else if (row < a.size0) {
 #pragma unroll
           for (int i = 0; i < EPV; ++i)
-            if (col + i < a.size1) ((elem_t*)g)[i] = ((const elem_t*)l)[i];
+            if (col + i < a.size1) ((elem_t*)g)[i] = regs[u].elem[i];
         }
       }
     }
+  };
+
+  union TiledVec {
+    uint4 vec;
+    piece_t piece[PIECES];
   };
 
   // ---- tiled side <-> LDS ----
   auto tiled_phase = [&]() {
-    const int32_t total = block_elems / VE;
-    for (int32_t v = tid; v < total; v += 256) {
-      const int32_t e = v * VE;
-      const TiledCoord c0 = tiled_coord(a, e, tile0_base, tile1_base);
-      if (!c0.in_range) continue;
-      union { uint4 vec; piece_t piece[PIECES]; } u;
-      if constexpr (!UNPACK) {
-        if constexpr (PIECES == 1) {
-          u.vec = *(const uint4*)(lds + c0.row * a.pitch_bytes + c0.col * E);
-        } else {
+    TiledVec regs[TILED_PER_THREAD];
+    TiledCoord first[TILED_PER_THREAD];
 #pragma unroll
-          for (int q = 0; q < PIECES; ++q) {
-            const TiledCoord c = tiled_coord(a, e + q * PL, tile0_base, tile1_base);
-            u.piece[q] = *(const piece_t*)(lds + c.row * a.pitch_bytes + c.col * E);
-          }
-        }
-        *(uint4*)(a.dst + c0.global_elem * E) = u.vec;
-      } else {
-        u.vec = *(const uint4*)(a.src + c0.global_elem * E);
-        if constexpr (PIECES == 1) {
-          *(uint4*)(lds + c0.row * a.pitch_bytes + c0.col * E) = u.vec;
-        } else {
-#pragma unroll
-          for (int q = 0; q < PIECES; ++q) {
-            const TiledCoord c = tiled_coord(a, e + q * PL, tile0_base, tile1_base);
-            *(piece_t*)(lds + c.row * a.pitch_bytes + c.col * E) = u.piece[q];
-          }
-        }
+    for (int u = 0; u < TILED_PER_THREAD; ++u) {
+      const int32_t e = (tid + 256 * u) * VE;
+      first[u] = tiled_coord(a, e, tile0_base, tile1_base);
+      if constexpr (UNPACK) {
+        if (first[u].in_range) regs[u].vec = *(const uint4*)(a.src + first[u].global_elem * E);
       }
+    }
+#pragma unroll
+    for (int u = 0; u < TILED_PER_THREAD; ++u) {
+      if (!first[u].in_range) continue;
+      const int32_t e = (tid + 256 * u) * VE;
+#pragma unroll
+      for (int q = 0; q < PIECES; ++q) {
+        int32_t row = first[u].row, col = first[u].col;
+        if (q > 0) {
+          const TiledCoord c = tiled_coord(a, e + q * PL, tile0_base, tile1_base);
+          row = c.row;
+          col = c.col;
+        }
+        piece_t* l = (piece_t*)(lds + row * a.pitch_bytes + col * E);
+        if constexpr (UNPACK) *l = regs[u].piece[q]; else regs[u].piece[q] = *l;
+      }
+      if constexpr (!UNPACK) *(uint4*)(a.dst + first[u].global_elem * E) = regs[u].vec;
     }
   };
 
   if constexpr (!UNPACK) {
-    flat_phase();
+    flat_load_phase();
     __syncthreads();
     tiled_phase();
   } else {
     tiled_phase();
     __syncthreads();
-    flat_phase();
+    flat_store_phase();
   }
 }
 
@@ -267,13 +315,13 @@ struct Plan {
 bool make_plan(const uint8_t* flat, const uint8_t* tiled, int64_t flat_stride0, int64_t flat_stride1,
                int64_t tiled_stride0, int64_t size0, int64_t size1, int64_t tsize0, int64_t tsize1,
                int64_t tsize2, int64_t tsize3, bool tr_inner, bool tr_outer, int elem_bytes,
-               Plan* plan) {
+               bool for_unpack, Plan* plan) {
   if (flat_stride1 != 1) return false;
   const int l2 = log2_exact(tsize2), l3 = log2_exact(tsize3);
   if (l2 < 0 || l3 < 0) return false;
   const int64_t tile_bytes = tsize2 * tsize3 * elem_bytes;
   if (tile_bytes % 16 || tile_bytes > 16384) return false;
-  if ((uintptr_t)tiled % 16 || (tiled_stride0 * elem_bytes) % 16) return false;
+  if ((uintptr_t)tiled % 16 || (tsize0 > 1 && (tiled_stride0 * elem_bytes) % 16)) return false;
   if ((uintptr_t)flat % elem_bytes) return false;
   if (size0 <= 0 || size1 <= 0) return false;  // nothing but padding: generic
 
@@ -291,35 +339,43 @@ bool make_plan(const uint8_t* flat, const uint8_t* tiled, int64_t flat_stride0, 
   a.size1 = size1;
   const int64_t T0 = 1ll << a.log2_t0, T1 = 1ll << a.log2_t1;
 
-  // Block shape: rows of at least 256 bytes on the 2-D side, runs of at least
-  // 1 KiB on the tiled side, about 16 KiB per block.
+  // Block shape: kBlockBytes of the 2-D matrix. Without an outer transpose one
+  // tile row (the tiled side is then a single contiguous run); with it, rows
+  // of at least 256 bytes and as many of them as fit (runs grow with rows).
   const int E = elem_bytes;
-  int64_t bc = 256 / E, br = T0;
-  if (bc < T1) bc = T1;
+  int64_t br, bc;
   if (!tr_outer) {
-    while (bc * T0 * E < 1024) bc *= 2;
+    br = T0;
+    bc = kBlockBytes / (br * E);
   } else {
-    while (br * T1 * E < 1024) br *= 2;
+    bc = 256 / E;
+    if (bc < T1) bc = T1;
+    br = kBlockBytes / (bc * E);
   }
-  while (br * bc * E < 16384) {
-    // Grow the dimension that lengthens the runs first, then the other.
-    if (!tr_outer) { if (bc * E < 2048) bc *= 2; else br *= 2; }
-    else { if (br * T1 * E < 4096) br *= 2; else bc *= 2; }
-  }
-  while (br * bc * E > 32768 && br > T0) br /= 2;
-  while (br * bc * E > 32768 && bc > T1 && bc * E > 256) bc /= 2;
-  if (br * bc * E > 49152) return false;
+  if (br < T0 || bc < T1 || br * bc * E != kBlockBytes) return false;
   a.log2_br = log2_exact(br);
   a.log2_bc = log2_exact(bc);
 
-  // Vector width on the 2-D side from the alignment shared by all rows.
-  int w = largest_pow2_dividing((uintptr_t)flat, 16);
+  // Vector width on the 2-D side from the alignment shared by all rows:
+  // 16-byte vectors need 4-byte alignment only.
+  int w = largest_pow2_dividing((uintptr_t)flat, 4);
   if (size0 > 1) {
-    const int ws = largest_pow2_dividing((uint64_t)(flat_stride0 * E), 16);
+    const int ws = largest_pow2_dividing((uint64_t)(flat_stride0 * E), 4);
     w = ws < w ? ws : w;
   }
-  if (w < E) w = E;
-  plan->flat_vec_bytes = w;
+  if (w < E) return false;
+  // Loads may be under-aligned 16-byte vectors; stores are faster when aligned,
+  // so unpack uses the widest vector that the rows are aligned to.
+  if (!for_unpack) {
+    plan->flat_vec_bytes = w == 4 ? 16 : w;
+  } else {
+    int wa = largest_pow2_dividing((uintptr_t)flat, 16);
+    if (size0 > 1) {
+      const int ws = largest_pow2_dividing((uint64_t)(flat_stride0 * E), 16);
+      wa = ws < wa ? ws : wa;
+    }
+    plan->flat_vec_bytes = wa;
+  }
 
   // Contiguous LDS piece on the tiled side.
   int piece = tr_inner ? E : (int)((T1 * E) < 16 ? (T1 * E) : 16);
@@ -334,9 +390,10 @@ bool make_plan(const uint8_t* flat, const uint8_t* tiled, int64_t flat_stride0, 
   const int64_t blocks0 = (rows_needed + br - 1) / br;
   a.blocks1 = (int32_t)((cols_needed + bc - 1) / bc);
   if (blocks0 * a.blocks1 >= (1ll << 31)) return false;
-  plan->grid = (unsigned)(blocks0 * a.blocks1);
+  a.total_blocks = (int32_t)(blocks0 * a.blocks1);
+  plan->grid = (unsigned)(((a.total_blocks + 7) / 8) * 8);
   plan->lds_bytes = (size_t)br * a.pitch_bytes;
-  return plan->lds_bytes <= 65536;
+  return plan->lds_bytes <= 49152;
 }
 
 template <int E, int W, bool UNPACK>
@@ -392,7 +449,7 @@ hipError_t launch_pack(const PackArgs& a, hipStream_t stream, const char** name)
   const bool tr_outer = a.flags & IREE_UK_FLAG_PACK_TRANSPOSE_OUTER;
   if (!make_plan(a.in, a.out, a.in_stride0, a.in_stride1, a.out_stride0, a.in_size0, a.in_size1,
                  a.out_size0, a.out_size1, a.out_size2, a.out_size3, tr_inner, tr_outer,
-                 a.elem_bytes, &plan))
+                 a.elem_bytes, /*for_unpack=*/false, &plan))
     return launch_pack_generic(a, stream, name);
   plan.args.src = a.in;
   plan.args.dst = a.out;
@@ -407,7 +464,7 @@ hipError_t launch_unpack(const UnpackArgs& a, hipStream_t stream, const char** n
   const bool tr_outer = a.flags & IREE_UK_FLAG_UNPACK_TRANSPOSE_OUTER;
   if (!make_plan(a.out, a.in, a.out_stride0, a.out_stride1, a.in_stride0, a.out_size0, a.out_size1,
                  a.in_size0, a.in_size1, a.in_size2, a.in_size3, tr_inner, tr_outer, a.elem_bytes,
-                 &plan))
+                 /*for_unpack=*/true, &plan))
     return launch_unpack_generic(a, stream, name);
   plan.args.src = a.in;
   plan.args.dst = a.out;
