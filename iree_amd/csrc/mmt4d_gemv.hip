@@ -1,0 +1,220 @@
+// mmt4d for skinny left-hand sides (at most 16 lhs rows in total, e.g. the
+// LLM decode shapes M0 in {1, 4, 16} with M = 1): an HBM-bandwidth kernel.
+//
+// Every rhs element is used exactly once, so the rhs streams from global memory
+// straight into MFMA operand registers, no LDS: for N0 = 16 a wavefront's
+// 16-row x 64-byte operand (lane l: row l & 15, 16-byte column l >> 4) covers
+// whole consecutive k steps of one tile, i.e. each load instruction reads 1 KiB
+// of contiguous memory. The (small, L2-resident) lhs is loaded the same way and
+// shared by the TN rhs tiles a wavefront works on. The wavefronts of a
+// workgroup split K between them and reduce through LDS in a fixed order, so
+// results do not depend on scheduling. The matrix pipe is mostly idle here by
+// design; it is used because its operand layout matches the tiled rhs exactly
+// and it keeps the VALU out of the inner loop.
+//
+// Covers s8s8s32, f16f16f32 and bf16bf16f32 with N0 = 16 and 16, 32 or 64
+// bytes per (k, row) piece.
+#include "uk_internal.h"
+
+namespace uk {
+namespace {
+
+typedef int v4i32 __attribute__((ext_vector_type(4)));
+typedef float v4f32 __attribute__((ext_vector_type(4)));
+typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
+typedef __bf16 v8bf16 __attribute__((ext_vector_type(8)));
+
+enum Kind { kI8 = 0, kF16 = 1, kBF16 = 2 };
+
+struct GemvArgs {
+  const uint8_t* lhs;
+  const uint8_t* rhs;
+  uint8_t* out;
+  int64_t lhs_stride_bytes, rhs_stride_bytes;
+  int64_t out_stride0;  // elements
+  int32_t M, N, K;
+  int32_t log2_M0;
+  int32_t rb, log2_rb;  // bytes of one (k, row) piece
+  int32_t steps;        // MFMA K-steps: ceil(K * rb / 64)
+  int32_t accumulate;
+};
+
+template <int KIND> struct Acc { typedef v4i32 type; };
+template <> struct Acc<kF16> { typedef v4f32 type; };
+template <> struct Acc<kBF16> { typedef v4f32 type; };
+
+template <int KIND>
+__device__ __forceinline__ typename Acc<KIND>::type mfma16(uint4 row_operand, uint4 col_operand,
+                                                           typename Acc<KIND>::type acc) {
+  if constexpr (KIND == kI8) {
+    return __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i32, row_operand),
+                                                 __builtin_bit_cast(v4i32, col_operand), acc, 0, 0, 0);
+  } else if constexpr (KIND == kF16) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, row_operand),
+                                                  __builtin_bit_cast(v8f16, col_operand), acc, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf16, row_operand),
+                                                   __builtin_bit_cast(v8bf16, col_operand), acc, 0, 0, 0);
+  }
+}
+
+// TN: rhs tiles per workgroup. UNROLL: K-steps whose loads are in flight together.
+template <int KIND, int TN, int UNROLL, int kWaves>
+__global__ __launch_bounds__(64 * kWaves) void mmt4d_gemv_kernel(const GemvArgs a) {
+  typedef typename Acc<KIND>::type acc_t;
+  __shared__ acc_t partial[kWaves][TN][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int row = lane & 15, g = lane >> 4;
+  const int32_t M0 = 1 << a.log2_M0;
+  const int32_t lhs_rows = a.M << a.log2_M0;  // <= 16
+
+  // Per-lane byte offset of its 16-byte operand column inside one K-step, as a
+  // function of the step: k1 = (64*step + 16*g) >> log2_rb.
+  const int32_t ksteps_per_step = 64 >> a.log2_rb;
+  const int32_t k1_lane = (16 * g) >> a.log2_rb;
+  const int32_t within = (16 * g) & (a.rb - 1);
+  const int64_t rhs_kstep = (int64_t)a.rb * 16;
+  const int64_t lhs_kstep = (int64_t)a.rb << a.log2_M0;
+
+  const bool lhs_valid = row < lhs_rows;
+  const uint8_t* lhs_lane = a.lhs + (int64_t)(row >> a.log2_M0) * a.lhs_stride_bytes +
+                            (int64_t)(row & (M0 - 1)) * a.rb + k1_lane * lhs_kstep + within;
+  const int64_t tile0 = (int64_t)blockIdx.x * TN;
+  const uint8_t* rhs_lane[TN];
+#pragma unroll
+  for (int t = 0; t < TN; ++t) {
+    const int64_t tile = tile0 + t < a.N ? tile0 + t : a.N - 1;  // clamp: computed, not stored
+    rhs_lane[t] = a.rhs + tile * a.rhs_stride_bytes + (int64_t)row * a.rb + k1_lane * rhs_kstep + within;
+  }
+
+  acc_t acc[TN];
+#pragma unroll
+  for (int t = 0; t < TN; ++t) acc[t] = acc_t{0, 0, 0, 0};
+
+  // This wavefront's share of the K-steps.
+  const int32_t per_wave = (a.steps + kWaves - 1) / kWaves;
+  const int32_t s_begin = wave * per_wave;
+  const int32_t s_end = min(s_begin + per_wave, a.steps);
+  // Steps whose k steps all lie below K need no checks.
+  const int32_t full_steps = a.K / ksteps_per_step;
+
+  int32_t s = s_begin;
+  for (; s + UNROLL <= min(s_end, full_steps); s += UNROLL) {
+    uint4 l[UNROLL], r[UNROLL][TN];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int64_t k1 = (int64_t)(s + u) * ksteps_per_step;
+      l[u] = make_uint4(0, 0, 0, 0);
+      if (lhs_valid) l[u] = *(const uint4*)(lhs_lane + k1 * lhs_kstep);
+#pragma unroll
+      for (int t = 0; t < TN; ++t) r[u][t] = __builtin_bit_cast(uint4, __builtin_nontemporal_load((const v4i32*)(rhs_lane[t] + k1 * rhs_kstep)));
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+      for (int t = 0; t < TN; ++t) acc[t] = mfma16<KIND>(r[u][t], l[u], acc[t]);
+  }
+  for (; s < s_end; ++s) {
+    const int64_t k1 = (int64_t)s * ksteps_per_step;
+    const bool in_k = k1 + k1_lane < a.K;
+    uint4 l = make_uint4(0, 0, 0, 0);
+    if (lhs_valid && in_k) l = *(const uint4*)(lhs_lane + k1 * lhs_kstep);
+#pragma unroll
+    for (int t = 0; t < TN; ++t) {
+      uint4 r = make_uint4(0, 0, 0, 0);
+      if (in_k) r = *(const uint4*)(rhs_lane[t] + k1 * rhs_kstep);
+      acc[t] = mfma16<KIND>(r, l, acc[t]);
+    }
+  }
+
+#pragma unroll
+  for (int t = 0; t < TN; ++t) partial[wave][t][lane] = acc[t];
+  __syncthreads();
+  if (wave != 0) return;
+  // Lane l holds lhs row l & 15 and rhs rows 4*(l >> 4) + {0..3} of each tile:
+  // four consecutive j0 of output row i0.
+  if (!lhs_valid) return;
+#pragma unroll
+  for (int t = 0; t < TN; ++t) {
+    if (tile0 + t >= a.N) continue;
+    acc_t v = partial[0][t][lane];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) v += partial[w][t][lane];
+    acc_t* dst = (acc_t*)(a.out + 4 * ((int64_t)(row >> a.log2_M0) * a.out_stride0 +
+                                       (tile0 + t) * ((int64_t)M0 * 16) +
+                                       (int64_t)(row & (M0 - 1)) * 16 + 4 * g));
+    if (a.accumulate) v += *dst;
+    *dst = v;
+  }
+}
+
+int log2_exact(int64_t v) {
+  if (v <= 0 || (v & (v - 1))) return -1;
+  int l = 0;
+  while ((1ll << l) < v) ++l;
+  return l;
+}
+
+bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, GemvArgs* g) {
+  int elem_bytes;
+  switch (a.flags & IREE_UK_FLAG_MMT4D_TYPE_MASK) {
+    case IREE_UK_FLAG_MMT4D_TYPE_S8S8S32: *kind = kI8; elem_bytes = 1; break;
+    case IREE_UK_FLAG_MMT4D_TYPE_F16F16F32: *kind = kF16; elem_bytes = 2; break;
+    case IREE_UK_FLAG_MMT4D_TYPE_BF16BF16F32: *kind = kBF16; elem_bytes = 2; break;
+    default: return false;
+  }
+  const int lm0 = log2_exact(a.M0);
+  const int rb = a.K0 * elem_bytes;
+  if (lm0 < 0 || a.M0 > 16 || a.N0 != 16) return false;
+  if (rb != 16 && rb != 32 && rb != 64) return false;
+  if (probe_only) return a.M0 < 16;  // 16-row tiles only when the whole lhs is that skinny
+  if (a.M * a.M0 > 16 || a.K == 0) return false;
+  // Worth it only when the rhs is long enough to stream.
+  if (a.N < 16) return false;
+  const int64_t lhs_stride_bytes = a.lhs_stride0 * elem_bytes;
+  const int64_t rhs_stride_bytes = a.rhs_stride0 * elem_bytes;
+  if ((uintptr_t)a.lhs % 16 || (a.M > 1 && lhs_stride_bytes % 16)) return false;
+  if ((uintptr_t)a.rhs % 16 || rhs_stride_bytes % 16) return false;
+  if ((uintptr_t)a.out % 16 || (a.M > 1 && a.out_stride0 % 4)) return false;
+  g->lhs = a.lhs; g->rhs = a.rhs; g->out = a.out;
+  g->lhs_stride_bytes = lhs_stride_bytes;
+  g->rhs_stride_bytes = rhs_stride_bytes;
+  g->out_stride0 = a.out_stride0;
+  g->M = (int32_t)a.M; g->N = (int32_t)a.N; g->K = (int32_t)a.K;
+  g->log2_M0 = lm0;
+  g->rb = rb;
+  g->log2_rb = log2_exact(rb);
+  g->steps = (int32_t)(((int64_t)a.K * rb + 63) / 64);
+  g->accumulate = (a.flags & IREE_UK_FLAG_MMT4D_ACCUMULATE) ? 1 : 0;
+  return true;
+}
+
+template <int KIND>
+hipError_t launch_kind(const GemvArgs& g, hipStream_t stream) {
+  // One rhs tile per workgroup (most workgroups, best balance over the CUs),
+  // 4 wavefronts splitting K, 16 KiB of rhs in flight per wavefront.
+  constexpr int TN = 1, UNROLL = 16, WAVES = 4;
+  hipLaunchKernelGGL((mmt4d_gemv_kernel<KIND, TN, UNROLL, WAVES>), dim3((g.N + TN - 1) / TN),
+                     dim3(64 * WAVES), 0, stream, g);
+  return hipGetLastError();
+}
+
+hipError_t launch_gemv(const Mmt4dArgs& a, hipStream_t stream, const char** name) {
+  int kind;
+  GemvArgs g;
+  if (!make_args(a, false, &kind, &g)) return hipErrorInvalidValue;
+  *name = "mmt4d_gemv";
+  if (kind == kI8) return launch_kind<kI8>(g, stream);
+  if (kind == kF16) return launch_kind<kF16>(g, stream);
+  return launch_kind<kBF16>(g, stream);
+}
+
+}  // namespace
+
+Mmt4dLauncher select_mmt4d_gemv(const Mmt4dArgs& a, bool probe_only) {
+  int kind;
+  GemvArgs g;
+  return make_args(a, probe_only, &kind, &g) ? launch_gemv : nullptr;
+}
+
+}  // namespace uk
