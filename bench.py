@@ -267,6 +267,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-also", action="store_true", help="headline workload only")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device-to-device copy three times (a kernel of "
+                         "known traffic, to scale the profiler's FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this library runs on ONE GPU (a ukernel call has no cross-device "
@@ -286,6 +289,13 @@ def main():
     head = _headline(torch, lib, abi, synth, args.steps, args.warmup)
     also = None if args.no_also else _also(torch, lib, abi, synth, max(6, args.steps // 5), 2)
     lib.iree_uk_mi355x_set_stream(None, 0)
+    if args.calibrate_copy:
+        a = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device="cuda").fill_(1)
+        b = torch.empty_like(a)
+        for _ in range(3):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        del a, b
 
     threads = min(16, os.cpu_count() or 1)
     cpu, cpu_arch = (None, None) if args.no_cpu else _cpu_baseline(abi, synth, threads)
