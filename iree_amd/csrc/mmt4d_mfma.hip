@@ -124,6 +124,94 @@ __device__ __forceinline__ uint4 load_piece(const uint8_t* p, int64_t kstep, int
   return v;
 }
 
+// Workgroup -> block tile. Consecutive workgroup ids go to different XCDs (8 of
+// them, each with its own L2), so ids are first regrouped so that one XCD works
+// on a contiguous range of tiles, then that range is walked in bands of 4 tile
+// rows so that neighbours share lhs and rhs panels. False: nothing to do.
+__device__ __forceinline__ bool locate_block(const MfmaArgs& a, int* tile_row, int* tile_col) {
+  const int total_tiles = a.tile_rows * a.tile_cols;
+  const int per_xcd = (total_tiles + 7) >> 3;
+  const int linear = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (linear >= total_tiles) return false;
+  constexpr int BAND = 4;
+  const int band = linear / (BAND * a.tile_cols);
+  const int band_first = band * BAND;
+  const int band_rows = min(a.tile_rows - band_first, BAND);
+  const int in_band = linear - band * BAND * a.tile_cols;
+  *tile_row = band_first + in_band % band_rows;
+  *tile_col = in_band / band_rows;
+  return true;
+}
+
+// Writes one wavefront's accumulators. Lane l holds, for fragment (i, j): lhs
+// row 32*i + (l & 31) and, in accumulator registers 4*q .. 4*q+3, rhs rows
+// 32*j + 8*q + 4*(l >> 5) + {0..3} of the wavefront's sub-block, which starts at
+// (wave_row, wave_col) of the logical matrix: four consecutive j0 of one output
+// row, one 128-bit store. When accumulating, all of a row's loads are issued
+// before the first add, so their latencies overlap.
+template <int KIND, bool RHS_I4, int AM, int BN>
+__device__ __forceinline__ void store_block(const MfmaArgs& a, typename AccType<KIND>::type (&acc)[AM][BN],
+                                            int64_t wave_row, int64_t wave_col, int lane) {
+  typedef typename AccType<KIND>::scalar scalar_t;
+  typedef scalar_t quad_t __attribute__((ext_vector_type(4)));
+  const int32_t M0 = 1 << a.log2_M0, N0 = 1 << a.log2_N0;
+  const int64_t total_rows = (int64_t)a.M << a.log2_M0;
+  const int64_t total_cols = (int64_t)a.N << a.log2_N0;
+  const int64_t row0 = wave_row + (lane & 31);
+  const int64_t col0 = wave_col + 4 * (lane >> 5);
+  // Byte offset of quad (j, q) from the sub-block's first column tile (the same
+  // for every row, and small) and whether the quad lies inside the matrix.
+  const int64_t first_col_tile = wave_col >> a.log2_N0;
+  uint8_t* wave_out = a.out + 4 * (first_col_tile << (a.log2_M0 + a.log2_N0));
+  uint32_t col_off[BN][4];
+  uint32_t col_inside = 0;
+#pragma unroll
+  for (int j = 0; j < BN; ++j)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int64_t col = col0 + 32 * j + 8 * q;
+      col_off[j][q] =
+          (uint32_t)(4 * ((((col >> a.log2_N0) - first_col_tile) << (a.log2_M0 + a.log2_N0)) + (col & (N0 - 1))));
+      if (col < total_cols) col_inside |= 1u << (4 * j + q);
+    }
+#pragma unroll
+  for (int i = 0; i < AM; ++i) {
+    const int64_t row = min(row0 + 32 * i, total_rows - 1);
+    const bool row_inside = row0 + 32 * i < total_rows;
+    uint8_t* row_out = wave_out + 4 * ((row >> a.log2_M0) * a.out_stride0 + ((row & (M0 - 1)) << a.log2_N0));
+#pragma unroll
+    for (int j = 0; j < BN; ++j) {
+      // Pin the fragment where it is until its turn: left alone, the compiler
+      // moves all 256 accumulators to ordinary registers right after the main
+      // loop, and there are not that many.
+      typename AccType<KIND>::type frag = acc[i][j];
+      asm volatile("" : "+a"(frag));
+      quad_t v[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        v[q] = quad_t{frag[4 * q], frag[4 * q + 1], frag[4 * q + 2], frag[4 * q + 3]};
+        if constexpr (RHS_I4) v[q] = v[q] >> 4;
+      }
+      if (a.accumulate) {
+        quad_t old[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          old[q] = quad_t{0, 0, 0, 0};
+          if (row_inside && (col_inside >> (4 * j + q) & 1)) old[q] = *(const quad_t*)(row_out + col_off[j][q]);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] += old[q];
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (row_inside && (col_inside >> (4 * j + q) & 1)) *(quad_t*)(row_out + col_off[j][q]) = v[q];
+      // Keep the fragments apart: hoisting all address arithmetic and
+      // accumulator reads to the top costs more registers than there are.
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+}
+
 template <int KIND, bool RHS_I4, int G, int AM, int BN, int MIN_BLOCKS, bool TAIL>
 __global__ __launch_bounds__(256, MIN_BLOCKS) void mmt4d_mfma_kernel(const MfmaArgs a) {
   typedef typename AccType<KIND>::type acc_t;
@@ -137,21 +225,8 @@ __global__ __launch_bounds__(256, MIN_BLOCKS) void mmt4d_mfma_kernel(const MfmaA
   __shared__ uint4 lds_a[2][A_PIECES];
   __shared__ uint4 lds_b[2][B_PIECES];
 
-  // Workgroup -> block tile. Consecutive workgroup ids go to different XCDs
-  // (8 of them, each with its own L2), so ids are first regrouped so that one
-  // XCD works on a contiguous range of tiles, then that range is walked in
-  // bands of 4 tile rows so that neighbours share lhs and rhs panels.
-  const int total_tiles = a.tile_rows * a.tile_cols;
-  const int per_xcd = (total_tiles + 7) >> 3;
-  const int linear = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (linear >= total_tiles) return;
-  constexpr int BAND = 4;
-  const int band = linear / (BAND * a.tile_cols);
-  const int band_first = band * BAND;
-  const int band_rows = min(a.tile_rows - band_first, BAND);
-  const int in_band = linear - band * BAND * a.tile_cols;
-  const int tile_row = band_first + in_band % band_rows;
-  const int tile_col = in_band / band_rows;
+  int tile_row, tile_col;
+  if (!locate_block(a, &tile_row, &tile_col)) return;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -344,35 +419,256 @@ __global__ __launch_bounds__(256, MIN_BLOCKS) void mmt4d_mfma_kernel(const MfmaA
     multiply(pa, pb, 1);
   }
 
-  // Epilogue. Lane l holds, for fragment (i, j): lhs row 32*i + (l & 31) and, in
-  // accumulator registers 4*q .. 4*q+3, rhs rows 32*j + 8*q + 4*(l >> 5) + {0..3}
-  // of the wavefront's sub-block: four consecutive j0 of one output row.
-  typedef typename AccType<KIND>::scalar scalar_t;
-  typedef scalar_t quad_t __attribute__((ext_vector_type(4)));
-  const int64_t row0 = first_row + wave_m * (32 * AM) + (lane & 31);
-  const int64_t col0 = first_col + wave_n * (32 * BN) + 4 * (lane >> 5);
-  const int64_t tile_elems = (int64_t)M0 * N0;
+  store_block<KIND, RHS_I4, AM, BN>(a, acc, first_row + wave_m * (32 * AM), first_col + wave_n * (32 * BN),
+                                    lane);
+}
+
+// ---------------------------------------------------------------------------
+// Direct-to-LDS variant: the same block tiling, but operand pieces travel
+// global memory -> LDS without passing through registers
+// (global_load_lds_dwordx4: lane l of a wavefront writes its 16 bytes at
+// M0 + 16*l), through a ring of 4 LDS stages filled three chunks ahead of the
+// MFMAs. It needs no register prefetch buffers, no LDS writes and no
+// data-dependent waits other than one counter wait per chunk. It covers the
+// int8/f16/bf16 rhs (no nibble widening on the way) and K that ends on a chunk
+// boundary; everything else uses the kernel above.
+//
+// Every load moves 16 contiguous bytes per lane, also for the 4-byte row
+// pieces of e.g. the 8x8x4 int8 tiles (G == 4), where 16 contiguous bytes are
+// 4 consecutive rows of one k step: there the transposition to "one row, 16
+// bytes of K" happens on the way out of LDS, with four 32-bit reads per
+// fragment instead of one 128-bit read, and the loads are arranged so that
+// those reads are linear in the lane number (conflict-free).
+//
+// The loads are issued from inline assembly: the compiler cannot see that they
+// write LDS, so it does not serialise the LDS reads against them; ordering is
+// enforced by hand with s_waitcnt vmcnt + a workgroup barrier once per chunk.
+extern __shared__ uint4 ring[];
+
+// One wavefront-wide load of 64 x 16 bytes to LDS byte offset `lds_off`
+// (wavefront-uniform) from `base` (uniform) + per-lane byte offset `voff`.
+__device__ __forceinline__ void load_to_lds(uint32_t lds_off, uint32_t voff, const uint8_t* base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_off), "v"(voff), "s"(base)
+               : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_loads_but() {
+  static_assert(N >= 0 && N <= 63, "vmcnt is a 6-bit counter");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+template <int KIND, int G, int AM, int BN, int MIN_BLOCKS>
+__global__ __launch_bounds__(256, MIN_BLOCKS) void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
+  typedef typename AccType<KIND>::type acc_t;
+  constexpr int BLOCK_ROWS = 64 * AM, BLOCK_COLS = 64 * BN;
+  constexpr int A_PIECES = BLOCK_ROWS * 4, B_PIECES = BLOCK_COLS * 4;  // 16-byte pieces per chunk
+  constexpr int STAGE_PIECES = A_PIECES + B_PIECES;
+  constexpr int STAGES = 4, AHEAD = 3;
+  // Load instructions per wavefront and chunk (64 lanes x 16 bytes each), each
+  // with its own per-lane offset.
+  constexpr int A_LOADS = A_PIECES / 256, B_LOADS = B_PIECES / 256;
+  constexpr int LOADS = A_LOADS + B_LOADS;
+  static_assert(A_PIECES % 256 == 0 && B_PIECES % 256 == 0, "block tile too small");
+  static_assert(2 * LOADS <= 63, "two chunks of loads must fit the 6-bit counter");
+
+  int tile_row, tile_col;
+  if (!locate_block(a, &tile_row, &tile_col)) return;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_m = wave >> 1, wave_n = wave & 1;
+
+  const int32_t M0 = 1 << a.log2_M0, N0 = 1 << a.log2_N0;
+  const int64_t total_rows = (int64_t)a.M << a.log2_M0;
+  const int64_t total_cols = (int64_t)a.N << a.log2_N0;
+  const int64_t lhs_kstep = (int64_t)a.lhs_rb << a.log2_M0;
+  const int64_t rhs_kstep = (int64_t)a.rhs_rb << a.log2_N0;
+  const int32_t ksteps_per_chunk = 64 >> a.log2_lhs_rb;
+  const int64_t lhs_chunk_bytes = ksteps_per_chunk * lhs_kstep;
+  const int64_t rhs_chunk_bytes = ksteps_per_chunk * rhs_kstep;
+
+  const int64_t first_row = (int64_t)tile_row * BLOCK_ROWS;
+  const int64_t first_col = (int64_t)tile_col * BLOCK_COLS;
+  const uint8_t* lhs_base = a.lhs + (first_row >> a.log2_M0) * a.lhs_stride_bytes;
+  const uint8_t* rhs_base = a.rhs + (first_col >> a.log2_N0) * a.rhs_stride_bytes;
+
+  // Load t of wavefront w fills the 16-byte LDS slots 64*m .. 64*m + 63 of its
+  // operand, m = 4*t + w, lane l the slot 64*m + l.
+  //   G == 16: slot p holds fragment p >> 7, 16-byte column (p >> 5) & 3 (K-step
+  //     c >> 1, lane half c & 1 of the MFMA operand), row p & 31: a fragment is
+  //     read back with one 128-bit read at slot 128*f + 64*kk + lane.
+  //   G == 4: slot 64*m + l holds rows 4*g .. 4*g + 3 (g = l & 7) of fragment
+  //     m >> 1 at k step 8*(m & 1) + 4*h + d of the chunk (h = (l >> 3) & 1,
+  //     d = l >> 4). Dword 64*(8*f + 4*kk + d) + 32*h + r of the operand is then
+  //     row r of fragment f at that k step: the MFMA operand of lane 32*h + r
+  //     for K-step kk is dwords d = 0..3, each read linear in the lane number.
+  //     K is permuted inside a chunk, identically for lhs and rhs.
+  // Rows past the end of the matrix are redirected to its last row (group):
+  // their products are computed, never stored.
+  auto row_offset = [&](int64_t row, int64_t last, int64_t first, int log2_t0, int64_t stride_bytes,
+                        int32_t rb) -> int64_t {
+    row = min(row, last);
+    const int64_t tile = (row >> log2_t0) - (first >> log2_t0);
+    return tile * stride_bytes + (row & ((1 << log2_t0) - 1)) * rb;
+  };
+  uint32_t a_off[A_LOADS], b_off[B_LOADS];
+  if constexpr (G == 16) {
 #pragma unroll
-  for (int i = 0; i < AM; ++i) {
-    const int64_t row = row0 + 32 * i;
-    if (row >= total_rows) continue;
-    const int64_t row_off = (row >> a.log2_M0) * a.out_stride0 + ((row & (M0 - 1)) << a.log2_N0);
-#pragma unroll
-    for (int j = 0; j < BN; ++j) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int64_t col = col0 + 32 * j + 8 * q;
-        if (col >= total_cols) continue;
-        quad_t* dst =
-            (quad_t*)(a.out + 4 * (row_off + (col >> a.log2_N0) * tile_elems + (col & (N0 - 1))));
-        quad_t v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
-                    acc[i][j][4 * q + 3]};
-        if constexpr (RHS_I4) v = v >> 4;
-        if (a.accumulate) v += *dst;
-        *dst = v;
-      }
+    for (int t = 0; t < A_LOADS; ++t) {
+      const int p = tid + 256 * t;
+      const int c = (p >> 5) & 3;
+      a_off[t] = (uint32_t)(row_offset(first_row + (p >> 7) * 32 + (p & 31), total_rows - 1, first_row,
+                                       a.log2_M0, a.lhs_stride_bytes, a.lhs_rb) +
+                            ((16 * c) >> a.log2_lhs_rb) * lhs_kstep + ((16 * c) & (a.lhs_rb - 1)));
     }
+#pragma unroll
+    for (int t = 0; t < B_LOADS; ++t) {
+      const int p = tid + 256 * t;
+      const int c = (p >> 5) & 3;
+      b_off[t] = (uint32_t)(row_offset(first_col + (p >> 7) * 32 + (p & 31), total_cols - 1, first_col,
+                                       a.log2_N0, a.rhs_stride_bytes, a.rhs_rb) +
+                            ((16 * c) >> a.log2_rhs_rb) * rhs_kstep + ((16 * c) & (a.rhs_rb - 1)));
+    }
+  } else {
+    const int g = lane & 7, k1 = 4 * ((lane >> 3) & 1) + (lane >> 4);
+#pragma unroll
+    for (int t = 0; t < A_LOADS; ++t)
+      a_off[t] = (uint32_t)(row_offset(first_row + 32 * (2 * t + (wave >> 1)) + 4 * g, total_rows - 4, first_row,
+                                       a.log2_M0, a.lhs_stride_bytes, a.lhs_rb) + k1 * lhs_kstep);
+#pragma unroll
+    for (int t = 0; t < B_LOADS; ++t)
+      b_off[t] = (uint32_t)(row_offset(first_col + 32 * (2 * t + (wave >> 1)) + 4 * g, total_cols - 4, first_col,
+                                       a.log2_N0, a.rhs_stride_bytes, a.rhs_rb) + k1 * rhs_kstep);
   }
+  // G == 4: this wavefront's loads all belong to K-step wave & 1.
+  const int64_t lhs_wave_bytes = G == 4 ? 8 * (wave & 1) * lhs_kstep : 0;
+  const int64_t rhs_wave_bytes = G == 4 ? 8 * (wave & 1) * rhs_kstep : 0;
+
+  acc_t acc[AM][BN];
+#pragma unroll
+  for (int i = 0; i < AM; ++i)
+#pragma unroll
+    for (int j = 0; j < BN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+
+  const int chunks = a.chunks;  // all full
+  const int last_chunk = chunks - 1;
+
+  // Load number `n` (compile-time after unrolling) of the chunk whose operand
+  // bases are la / lb, into the stage at LDS byte offset `stage_off`.
+  auto issue_load = [&](int n, uint32_t stage_off, const uint8_t* la, const uint8_t* lb) {
+    const bool is_a = n < A_LOADS;
+    const int t = is_a ? n : n - A_LOADS;
+    load_to_lds(stage_off + (is_a ? 0 : A_PIECES * 16) + (256 * t + 64 * wave) * 16,
+                is_a ? a_off[t] : b_off[t], is_a ? la : lb);
+  };
+  auto issue_chunk = [&](int kc) {
+    const int idx = min(kc, last_chunk);
+    const uint32_t stage_off = (uint32_t)(kc & (STAGES - 1)) * (STAGE_PIECES * 16);
+    const uint8_t* la = lhs_base + idx * lhs_chunk_bytes + lhs_wave_bytes;
+    const uint8_t* lb = rhs_base + idx * rhs_chunk_bytes + rhs_wave_bytes;
+#pragma unroll
+    for (int n = 0; n < LOADS; ++n) issue_load(n, stage_off, la, lb);
+  };
+
+  uint4 pa[AM][2], pb[BN][2], qa[AM][2], qb[BN][2];
+  // Fragment f of an operand at 16-byte slot `operand` of the ring, K-step kk.
+  auto read_frag = [&](int operand, int f, int kk) -> uint4 {
+    if constexpr (G == 16) {
+      return ring[operand + 128 * f + 64 * kk + lane];
+    } else {
+      const uint32_t* words = (const uint32_t*)(ring + operand) + 64 * (8 * f + 4 * kk) + lane;
+      return make_uint4(words[0], words[64], words[128], words[192]);
+    }
+  };
+  const int frag_a0 = wave_m * AM, frag_b0 = wave_n * BN;
+
+  // One pipeline step for chunk kc, whose fragments are in `cur`: wait until
+  // this wavefront's loads of chunk kc + 1 have landed, barrier (now everyone's
+  // have, and everyone is done reading the stage of chunk kc - 1), then the
+  // MFMAs of chunk kc with, between them, the loads of chunk kc + 3 into the
+  // stage just freed and the LDS reads of the fragments of chunk kc + 1.
+  //
+  // A wavefront issues in order and a memory instruction takes several cycles
+  // to issue, so more than one or two of them between two MFMAs lets the
+  // matrix pipe run dry: they are dealt out one (half) fragment and at most one
+  // load per MFMA. The reads go with the first three quarters of the MFMAs, so
+  // that the last of them has returned when the next step starts; fragments
+  // are read in the order the next step consumes them.
+  auto step = [&](int kc, const uint4 (*cur_a)[2], const uint4 (*cur_b)[2], uint4 (*nxt_a)[2],
+                  uint4 (*nxt_b)[2]) {
+    constexpr int MFMAS = 2 * AM * BN;
+    constexpr int PARTS = G == 4 ? 2 : 1;  // LDS read instructions per fragment (after pairing)
+    constexpr int READS = 2 * (AM + BN) * PARTS;
+    constexpr int READ_SLOTS = MFMAS >= 4 ? MFMAS * 3 / 4 : MFMAS;
+    wait_loads_but<LOADS*(AHEAD - 2)>();
+    __builtin_amdgcn_s_barrier();
+    const int load_kc = kc + AHEAD;
+    const int idx = min(load_kc, last_chunk);
+    const uint32_t load_stage_off = (uint32_t)(load_kc & (STAGES - 1)) * (STAGE_PIECES * 16);
+    const uint8_t* la = lhs_base + idx * lhs_chunk_bytes + lhs_wave_bytes;
+    const uint8_t* lb = rhs_base + idx * rhs_chunk_bytes + rhs_wave_bytes;
+    const int read_stage = ((kc + 1) & (STAGES - 1)) * STAGE_PIECES;
+#pragma unroll
+    for (int m = 0; m < MFMAS; ++m) {
+#pragma unroll
+      for (int n = m * LOADS / MFMAS; n < (m + 1) * LOADS / MFMAS; ++n) {
+        issue_load(n, load_stage_off, la, lb);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (m < READ_SLOTS) {
+#pragma unroll
+        for (int u = m * READS / READ_SLOTS; u < (m + 1) * READS / READ_SLOTS; ++u) {
+          const int f = u / PARTS, part = u % PARTS;
+          const int kk = f / (AM + BN), e = f % (AM + BN);
+          uint4& dst = e < BN ? nxt_b[e][kk] : nxt_a[e - BN][kk];
+          const int operand = e < BN ? read_stage + A_PIECES : read_stage;
+          const int frag = e < BN ? frag_b0 + e : frag_a0 + e - BN;
+          if constexpr (G == 16) {
+            dst = ring[operand + 128 * frag + 64 * kk + lane];
+          } else {
+            const uint32_t* words = (const uint32_t*)(ring + operand) + 64 * (8 * frag + 4 * kk + 2 * part) + lane;
+            if (part == 0) { dst.x = words[0]; dst.y = words[64]; }
+            else { dst.z = words[0]; dst.w = words[64]; }
+          }
+        }
+      }
+      {
+        const int kk = m / (AM * BN), i = (m % (AM * BN)) / BN, j = m % BN;
+        acc[i][j] = mfma<KIND>(cur_b[j][kk], cur_a[i][kk], acc[i][j]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  issue_chunk(0);
+  issue_chunk(1);
+  issue_chunk(2);
+  wait_loads_but<2 * LOADS>();
+  __syncthreads();
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+    for (int j = 0; j < BN; ++j) pb[j][kk] = read_frag(A_PIECES, frag_b0 + j, kk);
+#pragma unroll
+    for (int i = 0; i < AM; ++i) pa[i][kk] = read_frag(0, frag_a0 + i, kk);
+  }
+  int kc = 0;
+  for (; kc + 1 < chunks; kc += 2) {
+    step(kc, pa, pb, qa, qb);
+    step(kc + 1, qa, qb, pa, pb);
+  }
+  if (kc < chunks) step(kc, pa, pb, qa, qb);
+  // No load may still be writing LDS when the workgroup's allocation is freed.
+  wait_loads_but<0>();
+
+  store_block<KIND, false, AM, BN>(a, acc, first_row + wave_m * (32 * AM), first_col + wave_n * (32 * BN),
+                                   lane);
 }
 
 int log2_exact(int64_t v) {
@@ -463,6 +759,25 @@ hipError_t launch_tile(MfmaArgs m, hipStream_t stream) {
   const unsigned grid = (unsigned)(((tiles + 7) / 8) * 8);
   // K ending inside a chunk needs the kernel variant with the zero-filling tail step.
   const bool tail = ((int64_t)m.K * m.lhs_rb) % 64 != 0;
+  if constexpr (!RHS_I4) {
+    // 4-byte row pieces are loaded 4 rows (16 contiguous bytes) at a time there.
+    const bool rows_by_4 =
+        G == 16 || (m.log2_M0 >= 2 && m.log2_N0 >= 2 && (uintptr_t)m.lhs % 16 == 0 && (uintptr_t)m.rhs % 16 == 0 &&
+                    m.lhs_stride_bytes % 16 == 0 && m.rhs_stride_bytes % 16 == 0);
+    if (!tail && rows_by_4) {
+      // Ring of 4 stages in dynamic LDS; above 64 KiB the limit has to be raised
+      // (per device, so it is simply done on every launch: it only sets a field).
+      constexpr size_t lds_bytes = 4 * (64 * AM + 64 * BN) * 64;
+      auto kernel = mmt4d_mfma_direct_kernel<KIND, G, AM, BN, MIN_BLOCKS>;
+      if (lds_bytes > 65536) {
+        const hipError_t attr = hipFuncSetAttribute(
+            (const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (attr != hipSuccess) return attr;
+      }
+      hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds_bytes, stream, m);
+      return hipGetLastError();
+    }
+  }
   if (tail) {
     hipLaunchKernelGGL((mmt4d_mfma_kernel<KIND, RHS_I4, G, AM, BN, MIN_BLOCKS, true>), dim3(grid),
                        dim3(256), 0, stream, m);
