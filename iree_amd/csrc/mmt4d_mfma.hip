@@ -9,23 +9,29 @@
 // is walked in chunks of 64 BYTES per operand row (64 int8 or 32 f16/bf16
 // values = two MFMA K-steps).
 //
-// Data flow per chunk: global -> registers (issued two chunks ahead) -> LDS,
-// stored fragment-major so that a wavefront fetches one 32-row x 32-byte MFMA
-// operand with a single conflict-free 128-bit LDS read per lane -> registers
-// (read one chunk ahead) -> MFMA.
+// Two kernels share this tiling and the epilogue:
+//   mmt4d_mfma_direct_kernel (the fast path): operands go global memory ->
+//     LDS directly, 16 contiguous bytes per lane, through a ring of LDS stages
+//     filled several chunks ahead; needs K to end on a chunk boundary and
+//     16-byte aligned operand rows.
+//   mmt4d_mfma_kernel (everything else the plan admits: ragged K, 4-byte
+//     aligned operands, narrow tiles): global -> registers (issued two chunks
+//     ahead) -> LDS -> registers (read one chunk ahead) -> MFMA.
+// In both, LDS holds the operands fragment-major, so that a wavefront fetches
+// a 32-row x 32-byte MFMA operand with conflict-free reads that are linear in
+// the lane number.
 //
 // Operand layouts. An mmt4d operand row (one i0 of one tile) is not contiguous
 // in memory: its K0 values of consecutive k are M0*K0 elements apart
 // (mmt4d_tile_generic.c:70-71). With RB = bytes of one (k, i0) row piece:
-//   RB multiple of 16: a lane's 16 operand bytes are contiguous in memory and
-//     K is consumed in its natural order;
-//   RB == 4 (the 8x8x4 int8 tiles): a lane's 16 bytes are gathered from 4
-//     consecutive k steps. That permutes K inside a chunk, identically for
-//     lhs and rhs, which leaves every integer sum unchanged.
-// The int4 rhs of s8s4s32 is widened in registers on its way to LDS: nibble n
-// becomes the int8 value 16*n (sign in bit 7, no sign-extension step), the
-// accumulators therefore hold 16x the result and are shifted right by 4 at
-// the end, which is exact while 16*128*8*depth < 2^31.
+//   RB multiple of 16: a lane's 16 operand bytes are contiguous in memory;
+//   RB == 4 (the 8x8x4 int8 tiles): a lane's 16 bytes come from 4 different k
+//     steps. K is permuted inside a chunk, identically for lhs and rhs, which
+//     leaves every integer sum unchanged (and reorders a float sum).
+// The int4 rhs of s8s4s32 is widened in registers: nibble n becomes the int8
+// value 16*n (sign in bit 7, no sign-extension step), the accumulators
+// therefore hold 16x the result and are shifted right by 4 at the end, which
+// is exact while 16*128*8*depth < 2^31.
 //
 // The MFMA is issued with the rhs fragment as its row operand and the lhs
 // fragment as its column operand, so a lane ends up with 4 consecutive j0 of
@@ -80,17 +86,17 @@ __device__ __forceinline__ typename AccType<KIND>::type mfma(uint4 row_operand, 
 }
 
 // 16 int4 values (two dwords, element 2b in the low nibble of byte b) to 16
-// int8 values equal to 16x the signed nibbles, in element order.
+// int8 values equal to 16x the signed nibbles, in element order: the even and
+// the odd elements of a dword are isolated in the high nibbles of two dwords,
+// whose bytes are then interleaved.
 __device__ __forceinline__ uint4 widen_i4_times16(uint2 w) {
-  const uint32_t lo0 = (w.x << 4) & 0xF0F0F0F0u, hi0 = w.x & 0xF0F0F0F0u;
-  const uint32_t lo1 = (w.y << 4) & 0xF0F0F0F0u, hi1 = w.y & 0xF0F0F0F0u;
+  const uint32_t even0 = (w.x << 4) & 0xF0F0F0F0u, odd0 = w.x & 0xF0F0F0F0u;
+  const uint32_t even1 = (w.y << 4) & 0xF0F0F0F0u, odd1 = w.y & 0xF0F0F0F0u;
   uint4 r;
-  r.x = (lo0 & 0xFFu) | ((hi0 & 0xFFu) << 8) | ((lo0 & 0xFF00u) << 8) | ((hi0 & 0xFF00u) << 16);
-  r.y = ((lo0 >> 16) & 0xFFu) | (((hi0 >> 16) & 0xFFu) << 8) | ((lo0 >> 8) & 0xFF0000u) |
-        (hi0 & 0xFF000000u);
-  r.z = (lo1 & 0xFFu) | ((hi1 & 0xFFu) << 8) | ((lo1 & 0xFF00u) << 8) | ((hi1 & 0xFF00u) << 16);
-  r.w = ((lo1 >> 16) & 0xFFu) | (((hi1 >> 16) & 0xFFu) << 8) | ((lo1 >> 8) & 0xFF0000u) |
-        (hi1 & 0xFF000000u);
+  r.x = __builtin_amdgcn_perm(odd0, even0, 0x05010400u);
+  r.y = __builtin_amdgcn_perm(odd0, even0, 0x07030602u);
+  r.z = __builtin_amdgcn_perm(odd1, even1, 0x05010400u);
+  r.w = __builtin_amdgcn_perm(odd1, even1, 0x07030602u);
   return r;
 }
 
@@ -460,19 +466,26 @@ __device__ __forceinline__ void wait_loads_but() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-template <int KIND, int G, int AM, int BN, int MIN_BLOCKS>
-__global__ __launch_bounds__(256, MIN_BLOCKS) void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
+template <int KIND, bool RHS_I4, int G, int AM, int BN, int STAGES>
+__global__ __launch_bounds__(256) void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   typedef typename AccType<KIND>::type acc_t;
+  static_assert(!RHS_I4 || (G == 16 && BN >= 2), "int4 rhs: 16-byte pieces, at least one fragment per wavefront");
   constexpr int BLOCK_ROWS = 64 * AM, BLOCK_COLS = 64 * BN;
-  constexpr int A_PIECES = BLOCK_ROWS * 4, B_PIECES = BLOCK_COLS * 4;  // 16-byte pieces per chunk
-  constexpr int STAGE_PIECES = A_PIECES + B_PIECES;
-  constexpr int STAGES = 4, AHEAD = 3;
+  // 16-byte pieces per chunk: 64 bytes of K per row, 32 bytes for an int4 rhs.
+  constexpr int A_PIECES = BLOCK_ROWS * 4, B_PIECES = BLOCK_COLS * (RHS_I4 ? 2 : 4);
+  // Stage size rounded up to a power of two so that ring offsets wrap with a mask.
+  constexpr int STAGE_PIECES = A_PIECES + B_PIECES <= 512    ? 512
+                               : A_PIECES + B_PIECES <= 1024 ? 1024
+                                                             : 2048;
+  static_assert(A_PIECES + B_PIECES <= STAGE_PIECES, "stage too small");
+  constexpr int AHEAD = STAGES - 1;  // chunks in flight ahead of the one being multiplied
+  static_assert(STAGES >= 4 && (STAGES & (STAGES - 1)) == 0, "ring depth");
   // Load instructions per wavefront and chunk (64 lanes x 16 bytes each), each
   // with its own per-lane offset.
   constexpr int A_LOADS = A_PIECES / 256, B_LOADS = B_PIECES / 256;
   constexpr int LOADS = A_LOADS + B_LOADS;
   static_assert(A_PIECES % 256 == 0 && B_PIECES % 256 == 0, "block tile too small");
-  static_assert(2 * LOADS <= 63, "two chunks of loads must fit the 6-bit counter");
+  static_assert((AHEAD - 1) * LOADS <= 63, "the loads in flight must fit the 6-bit counter");
 
   int tile_row, tile_col;
   if (!locate_block(a, &tile_row, &tile_col)) return;
@@ -507,6 +520,10 @@ __global__ __launch_bounds__(256, MIN_BLOCKS) void mmt4d_mfma_direct_kernel(cons
   //     row r of fragment f at that k step: the MFMA operand of lane 32*h + r
   //     for K-step kk is dwords d = 0..3, each read linear in the lane number.
   //     K is permuted inside a chunk, identically for lhs and rhs.
+  //   int4 rhs: slot 64*f + 32*h + r holds nibbles 32*h .. 32*h + 31 of row r of
+  //     fragment f: lane 32*h + r reads that slot once per chunk and widens its
+  //     first 8 bytes for K-step 0, its last 8 for K-step 1. The lhs columns are
+  //     assigned to match: (K-step kk, lane half h) gets 16-byte column kk + 2*h.
   // Rows past the end of the matrix are redirected to its last row (group):
   // their products are computed, never stored.
   auto row_offset = [&](int64_t row, int64_t last, int64_t first, int log2_t0, int64_t stride_bytes,
@@ -520,7 +537,7 @@ __global__ __launch_bounds__(256, MIN_BLOCKS) void mmt4d_mfma_direct_kernel(cons
 #pragma unroll
     for (int t = 0; t < A_LOADS; ++t) {
       const int p = tid + 256 * t;
-      const int c = (p >> 5) & 3;
+      const int c = RHS_I4 ? ((p >> 6) & 1) + 2 * ((p >> 5) & 1) : (p >> 5) & 3;
       a_off[t] = (uint32_t)(row_offset(first_row + (p >> 7) * 32 + (p & 31), total_rows - 1, first_row,
                                        a.log2_M0, a.lhs_stride_bytes, a.lhs_rb) +
                             ((16 * c) >> a.log2_lhs_rb) * lhs_kstep + ((16 * c) & (a.lhs_rb - 1)));
@@ -528,9 +545,10 @@ __global__ __launch_bounds__(256, MIN_BLOCKS) void mmt4d_mfma_direct_kernel(cons
 #pragma unroll
     for (int t = 0; t < B_LOADS; ++t) {
       const int p = tid + 256 * t;
-      const int c = (p >> 5) & 3;
-      b_off[t] = (uint32_t)(row_offset(first_col + (p >> 7) * 32 + (p & 31), total_cols - 1, first_col,
-                                       a.log2_N0, a.rhs_stride_bytes, a.rhs_rb) +
+      const int c = RHS_I4 ? (p >> 5) & 1 : (p >> 5) & 3;
+      const int row = RHS_I4 ? (p >> 6) * 32 + (p & 31) : (p >> 7) * 32 + (p & 31);
+      b_off[t] = (uint32_t)(row_offset(first_col + row, total_cols - 1, first_col, a.log2_N0,
+                                       a.rhs_stride_bytes, a.rhs_rb) +
                             ((16 * c) >> a.log2_rhs_rb) * rhs_kstep + ((16 * c) & (a.rhs_rb - 1)));
     }
   } else {
@@ -579,6 +597,10 @@ __global__ __launch_bounds__(256, MIN_BLOCKS) void mmt4d_mfma_direct_kernel(cons
   uint4 pa[AM][2], pb[BN][2], qa[AM][2], qb[BN][2];
   // Fragment f of an operand at 16-byte slot `operand` of the ring, K-step kk.
   auto read_frag = [&](int operand, int f, int kk) -> uint4 {
+    if (RHS_I4 && operand >= A_PIECES) {
+      const uint4 raw = ring[operand + 64 * f + lane];
+      return widen_i4_times16(kk ? make_uint2(raw.z, raw.w) : make_uint2(raw.x, raw.y));
+    }
     if constexpr (G == 16) {
       return ring[operand + 128 * f + 64 * kk + lane];
     } else {
@@ -588,68 +610,119 @@ __global__ __launch_bounds__(256, MIN_BLOCKS) void mmt4d_mfma_direct_kernel(cons
   };
   const int frag_a0 = wave_m * AM, frag_b0 = wave_n * BN;
 
-  // One pipeline step for chunk kc, whose fragments are in `cur`: wait until
-  // this wavefront's loads of chunk kc + 1 have landed, barrier (now everyone's
-  // have, and everyone is done reading the stage of chunk kc - 1), then the
-  // MFMAs of chunk kc with, between them, the loads of chunk kc + 3 into the
-  // stage just freed and the LDS reads of the fragments of chunk kc + 1.
-  //
+  // Loop-carried, wavefront-uniform state: where the next chunk to load comes
+  // from and goes to, and the stage the next fragments are read from. Kept as
+  // running values (a few scalar adds per step) rather than recomputed from the
+  // chunk number (64-bit multiplies on the scalar unit, in front of the step's
+  // first MFMA).
+  constexpr uint32_t STAGE_BYTES = STAGE_PIECES * 16, RING_BYTES = STAGES * STAGE_BYTES;
+  static_assert((RING_BYTES & (RING_BYTES - 1)) == 0, "ring offsets wrap with a mask");
+  const uint8_t* load_a = lhs_base + min(AHEAD, last_chunk) * lhs_chunk_bytes + lhs_wave_bytes;
+  const uint8_t* load_b = rhs_base + min(AHEAD, last_chunk) * rhs_chunk_bytes + rhs_wave_bytes;
+  int load_chunk = AHEAD;
+  uint32_t load_stage_off = AHEAD * STAGE_BYTES % RING_BYTES;
+  uint32_t read_stage_off = STAGE_BYTES;
+  const uint32_t frag_a_off = (uint32_t)((wave_m * AM) * 128) * 16;
+  const uint32_t frag_b_off = (uint32_t)(A_PIECES + (wave_n * BN) * (RHS_I4 ? 64 : 128)) * 16;
+  const uint8_t* ring_bytes = (const uint8_t*)ring + (G == 16 ? 16 : 4) * lane;
+
+  // One pipeline step for the chunk whose fragments are in `cur`:
+  //   a few MFMAs first (they only need registers, and keep the matrix pipe
+  //   fed across the barrier); wait until this wavefront's loads of the next
+  //   chunk have landed; barrier (now everyone's have, and everyone is done
+  //   reading the stage of the previous chunk); then the remaining MFMAs with,
+  //   between them, the loads of the chunk three ahead into the stage just
+  //   freed and the LDS reads of the next chunk's fragments.
   // A wavefront issues in order and a memory instruction takes several cycles
   // to issue, so more than one or two of them between two MFMAs lets the
   // matrix pipe run dry: they are dealt out one (half) fragment and at most one
-  // load per MFMA. The reads go with the first three quarters of the MFMAs, so
-  // that the last of them has returned when the next step starts; fragments
-  // are read in the order the next step consumes them.
-  auto step = [&](int kc, const uint4 (*cur_a)[2], const uint4 (*cur_b)[2], uint4 (*nxt_a)[2],
-                  uint4 (*nxt_b)[2]) {
+  // load per MFMA. The reads end a quarter of the step before its end, so that
+  // the last of them has returned when the next step starts; fragments are
+  // read in the order the next step consumes them.
+  auto step = [&](const uint4 (*cur_a)[2], const uint4 (*cur_b)[2], uint4 (*nxt_a)[2], uint4 (*nxt_b)[2]) {
     constexpr int MFMAS = 2 * AM * BN;
     constexpr int PARTS = G == 4 ? 2 : 1;  // LDS read instructions per fragment (after pairing)
-    constexpr int READS = 2 * (AM + BN) * PARTS;
-    constexpr int READ_SLOTS = MFMAS >= 4 ? MFMAS * 3 / 4 : MFMAS;
+    // Read units, in the order the next step consumes them: per K-step the rhs
+    // fragments, then the lhs fragments. An int4 rhs fragment is read once, raw,
+    // for both K-steps (first), and widened after the last read has been issued.
+    constexpr int B_UNITS = RHS_I4 ? BN : 0;
+    constexpr int READS = RHS_I4 ? BN + 2 * AM : 2 * (AM + BN) * PARTS;
+    constexpr int LEAD = MFMAS >= 16 ? 4 : (MFMAS >= 8 ? 2 : 0);   // MFMAs ahead of the barrier
+    constexpr int TAIL_FREE = MFMAS >= 8 ? MFMAS / 4 : 0;          // MFMAs after the last read
+    constexpr int SLOTS = MFMAS - LEAD - TAIL_FREE;                // MFMAs that carry memory work
+    static_assert(SLOTS >= 1, "no room for the memory instructions");
+    static_assert(!RHS_I4 || TAIL_FREE >= 1, "nowhere to widen");
+    auto multiply = [&](int m) {
+      const int kk = m / (AM * BN), i = (m % (AM * BN)) / BN, j = m % BN;
+      acc[i][j] = mfma<KIND>(cur_b[j][kk], cur_a[i][kk], acc[i][j]);
+    };
+#pragma unroll
+    for (int m = 0; m < LEAD; ++m) multiply(m);
+    __builtin_amdgcn_sched_barrier(0);
     wait_loads_but<LOADS*(AHEAD - 2)>();
     __builtin_amdgcn_s_barrier();
-    const int load_kc = kc + AHEAD;
-    const int idx = min(load_kc, last_chunk);
-    const uint32_t load_stage_off = (uint32_t)(load_kc & (STAGES - 1)) * (STAGE_PIECES * 16);
-    const uint8_t* la = lhs_base + idx * lhs_chunk_bytes + lhs_wave_bytes;
-    const uint8_t* lb = rhs_base + idx * rhs_chunk_bytes + rhs_wave_bytes;
-    const int read_stage = ((kc + 1) & (STAGES - 1)) * STAGE_PIECES;
+    const uint8_t* read_a = ring_bytes + read_stage_off + frag_a_off;
+    const uint8_t* read_b = ring_bytes + read_stage_off + frag_b_off;
+    uint4 raw_b[RHS_I4 ? BN : 1];
 #pragma unroll
-    for (int m = 0; m < MFMAS; ++m) {
+    for (int m = LEAD; m < MFMAS; ++m) {
+      const int slot = m - LEAD;
+      if (slot < SLOTS) {
 #pragma unroll
-      for (int n = m * LOADS / MFMAS; n < (m + 1) * LOADS / MFMAS; ++n) {
-        issue_load(n, load_stage_off, la, lb);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      if (m < READ_SLOTS) {
+        for (int n = slot * LOADS / SLOTS; n < (slot + 1) * LOADS / SLOTS; ++n)
+          issue_load(n, load_stage_off, load_a, load_b);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int u = m * READS / READ_SLOTS; u < (m + 1) * READS / READ_SLOTS; ++u) {
-          const int f = u / PARTS, part = u % PARTS;
-          const int kk = f / (AM + BN), e = f % (AM + BN);
-          uint4& dst = e < BN ? nxt_b[e][kk] : nxt_a[e - BN][kk];
-          const int operand = e < BN ? read_stage + A_PIECES : read_stage;
-          const int frag = e < BN ? frag_b0 + e : frag_a0 + e - BN;
-          if constexpr (G == 16) {
-            dst = ring[operand + 128 * frag + 64 * kk + lane];
+        for (int u = slot * READS / SLOTS; u < (slot + 1) * READS / SLOTS; ++u) {
+          if constexpr (RHS_I4) {
+            if (u < B_UNITS) {
+              raw_b[u] = *(const uint4*)(read_b + (64 * u) * 16);
+            } else {
+              const int kk = (u - B_UNITS) / AM, i = (u - B_UNITS) % AM;
+              nxt_a[i][kk] = *(const uint4*)(read_a + (128 * i + 64 * kk) * 16);
+            }
           } else {
-            const uint32_t* words = (const uint32_t*)(ring + operand) + 64 * (8 * frag + 4 * kk + 2 * part) + lane;
-            if (part == 0) { dst.x = words[0]; dst.y = words[64]; }
-            else { dst.z = words[0]; dst.w = words[64]; }
+            const int f = u / PARTS, part = u % PARTS;
+            const int kk = f / (AM + BN), e = f % (AM + BN);
+            uint4& dst = e < BN ? nxt_b[e][kk] : nxt_a[e - BN][kk];
+            const uint8_t* src = e < BN ? read_b : read_a;
+            const int frag = e < BN ? e : e - BN;
+            if constexpr (G == 16) {
+              dst = *(const uint4*)(src + (128 * frag + 64 * kk) * 16);
+            } else {
+              const uint32_t* words = (const uint32_t*)src + 64 * (8 * frag + 4 * kk + 2 * part);
+              if (part == 0) { dst.x = words[0]; dst.y = words[64]; }
+              else { dst.z = words[0]; dst.w = words[64]; }
+            }
           }
         }
+      } else if constexpr (RHS_I4) {
+        // Widening, dealt out over the MFMAs that carry no memory work.
+        const int tail = slot - SLOTS;
+#pragma unroll
+        for (int w = tail * 2 * BN / TAIL_FREE; w < (tail + 1) * 2 * BN / TAIL_FREE; ++w) {
+          const int kk = w / BN, j = w % BN;
+          nxt_b[j][kk] = widen_i4_times16(kk ? make_uint2(raw_b[j].z, raw_b[j].w) : make_uint2(raw_b[j].x, raw_b[j].y));
+        }
       }
-      {
-        const int kk = m / (AM * BN), i = (m % (AM * BN)) / BN, j = m % BN;
-        acc[i][j] = mfma<KIND>(cur_b[j][kk], cur_a[i][kk], acc[i][j]);
+      multiply(m);
+      if (m == MFMAS - 1) {
+        // Advance the running state (clamped at the last chunk: the loads
+        // issued beyond it are redundant, their stages are never read).
+        const bool more = load_chunk < last_chunk;
+        load_a += more ? lhs_chunk_bytes : 0;
+        load_b += more ? rhs_chunk_bytes : 0;
+        ++load_chunk;
+        load_stage_off = (load_stage_off + STAGE_BYTES) & (RING_BYTES - 1);
+        read_stage_off = (read_stage_off + STAGE_BYTES) & (RING_BYTES - 1);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
   };
 
-  issue_chunk(0);
-  issue_chunk(1);
-  issue_chunk(2);
-  wait_loads_but<2 * LOADS>();
+#pragma unroll
+  for (int c = 0; c < AHEAD; ++c) issue_chunk(c);
+  wait_loads_but<(AHEAD - 1) * LOADS>();
   __syncthreads();
 #pragma unroll
   for (int kk = 0; kk < 2; ++kk) {
@@ -660,15 +733,15 @@ __global__ __launch_bounds__(256, MIN_BLOCKS) void mmt4d_mfma_direct_kernel(cons
   }
   int kc = 0;
   for (; kc + 1 < chunks; kc += 2) {
-    step(kc, pa, pb, qa, qb);
-    step(kc + 1, qa, qb, pa, pb);
+    step(pa, pb, qa, qb);
+    step(qa, qb, pa, pb);
   }
-  if (kc < chunks) step(kc, pa, pb, qa, qb);
+  if (kc < chunks) step(pa, pb, qa, qb);
   // No load may still be writing LDS when the workgroup's allocation is freed.
   wait_loads_but<0>();
 
-  store_block<KIND, false, AM, BN>(a, acc, first_row + wave_m * (32 * AM), first_col + wave_n * (32 * BN),
-                                   lane);
+  store_block<KIND, RHS_I4, AM, BN>(a, acc, first_row + wave_m * (32 * AM), first_col + wave_n * (32 * BN),
+                                    lane);
 }
 
 int log2_exact(int64_t v) {
@@ -750,34 +823,53 @@ bool make_plan(const Mmt4dArgs& a, bool probe_only, Plan* plan) {
   return true;
 }
 
+// Whether the direct-to-LDS kernel covers the problem: K ends on a chunk
+// boundary and every lane can load 16 contiguous bytes (4-byte row pieces 4
+// rows at a time, an int4 rhs in pieces of 32 nibbles).
+template <bool RHS_I4, int G>
+bool direct_covers(const MfmaArgs& m) {
+  if (((int64_t)m.K * m.lhs_rb) % 64 != 0) return false;
+  if (RHS_I4) return m.rhs_rb >= 16 && (uintptr_t)m.rhs % 16 == 0 && m.rhs_stride_bytes % 16 == 0;
+  if (G == 16) return true;
+  return m.log2_M0 >= 2 && m.log2_N0 >= 2 && (uintptr_t)m.lhs % 16 == 0 && (uintptr_t)m.rhs % 16 == 0 &&
+         m.lhs_stride_bytes % 16 == 0 && m.rhs_stride_bytes % 16 == 0;
+}
+
+void set_tile_grid(MfmaArgs* m, int block_rows, int block_cols, unsigned* grid) {
+  const int64_t rows = (int64_t)m->M << m->log2_M0, cols = (int64_t)m->N << m->log2_N0;
+  m->tile_rows = (int32_t)((rows + block_rows - 1) / block_rows);
+  m->tile_cols = (int32_t)((cols + block_cols - 1) / block_cols);
+  const int64_t tiles = (int64_t)m->tile_rows * m->tile_cols;
+  *grid = (unsigned)(((tiles + 7) / 8) * 8);
+}
+
+// Direct-to-LDS kernel on (64*AM) x (64*BN) block tiles with a ring of STAGES stages.
+template <int KIND, bool RHS_I4, int G, int AM, int BN, int STAGES>
+hipError_t launch_direct(MfmaArgs m, hipStream_t stream) {
+  unsigned grid;
+  set_tile_grid(&m, 64 * AM, 64 * BN, &grid);
+  constexpr int stage_pieces = 256 * AM + (RHS_I4 ? 128 : 256) * BN;
+  constexpr size_t lds_bytes = (size_t)STAGES * 16 * (stage_pieces <= 512 ? 512 : stage_pieces <= 1024 ? 1024 : 2048);
+  static_assert(lds_bytes <= 160 * 1024, "ring does not fit the LDS");
+  auto kernel = mmt4d_mfma_direct_kernel<KIND, RHS_I4, G, AM, BN, STAGES>;
+  // Above 64 KiB of dynamic LDS the limit has to be raised (per device, so it
+  // is simply done on every launch: it only sets a field).
+  if (lds_bytes > 65536) {
+    const hipError_t attr =
+        hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (attr != hipSuccess) return attr;
+  }
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds_bytes, stream, m);
+  return hipGetLastError();
+}
+
+// Register-staged kernel (any K, any alignment the plan admits).
 template <int KIND, bool RHS_I4, int G, int AM, int BN, int MIN_BLOCKS>
-hipError_t launch_tile(MfmaArgs m, hipStream_t stream) {
-  const int64_t rows = (int64_t)m.M << m.log2_M0, cols = (int64_t)m.N << m.log2_N0;
-  m.tile_rows = (int32_t)((rows + 64 * AM - 1) / (64 * AM));
-  m.tile_cols = (int32_t)((cols + 64 * BN - 1) / (64 * BN));
-  const int64_t tiles = (int64_t)m.tile_rows * m.tile_cols;
-  const unsigned grid = (unsigned)(((tiles + 7) / 8) * 8);
+hipError_t launch_staged(MfmaArgs m, hipStream_t stream) {
+  unsigned grid;
+  set_tile_grid(&m, 64 * AM, 64 * BN, &grid);
   // K ending inside a chunk needs the kernel variant with the zero-filling tail step.
   const bool tail = ((int64_t)m.K * m.lhs_rb) % 64 != 0;
-  if constexpr (!RHS_I4) {
-    // 4-byte row pieces are loaded 4 rows (16 contiguous bytes) at a time there.
-    const bool rows_by_4 =
-        G == 16 || (m.log2_M0 >= 2 && m.log2_N0 >= 2 && (uintptr_t)m.lhs % 16 == 0 && (uintptr_t)m.rhs % 16 == 0 &&
-                    m.lhs_stride_bytes % 16 == 0 && m.rhs_stride_bytes % 16 == 0);
-    if (!tail && rows_by_4) {
-      // Ring of 4 stages in dynamic LDS; above 64 KiB the limit has to be raised
-      // (per device, so it is simply done on every launch: it only sets a field).
-      constexpr size_t lds_bytes = 4 * (64 * AM + 64 * BN) * 64;
-      auto kernel = mmt4d_mfma_direct_kernel<KIND, G, AM, BN, MIN_BLOCKS>;
-      if (lds_bytes > 65536) {
-        const hipError_t attr = hipFuncSetAttribute(
-            (const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        if (attr != hipSuccess) return attr;
-      }
-      hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds_bytes, stream, m);
-      return hipGetLastError();
-    }
-  }
   if (tail) {
     hipLaunchKernelGGL((mmt4d_mfma_kernel<KIND, RHS_I4, G, AM, BN, MIN_BLOCKS, true>), dim3(grid),
                        dim3(256), 0, stream, m);
@@ -788,21 +880,30 @@ hipError_t launch_tile(MfmaArgs m, hipStream_t stream) {
   return hipGetLastError();
 }
 
-// Picks the largest block tile that still gives every compute unit work.
+// Picks the block tile. Every workgroup pulls its operands through L2 -> LDS at
+// a rate that does not depend on the tile, so the bytes moved per multiply
+// fall with the tile's size: the largest tile that still gives most compute
+// units a workgroup wins.
 template <int KIND, bool RHS_I4, int G>
 hipError_t launch_variant(const MfmaArgs& m, hipStream_t stream, const char** name) {
   const int64_t rows = (int64_t)m.M << m.log2_M0, cols = (int64_t)m.N << m.log2_N0;
   auto tiles = [&](int br, int bc) { return ((rows + br - 1) / br) * ((cols + bc - 1) / bc); };
+  const bool direct = direct_covers<RHS_I4, G>(m);
   if (tiles(256, 256) >= 200) {
     *name = "mmt4d_mfma_256x256";
-    return launch_tile<KIND, RHS_I4, G, 4, 4, 1>(m, stream);
+    if (direct) return launch_direct<KIND, RHS_I4, G, 4, 4, 4>(m, stream);
+    return launch_staged<KIND, RHS_I4, G, 4, 4, 1>(m, stream);
   }
-  if (tiles(128, 128) >= 200 || (rows > 64 && cols > 64)) {
+  if (tiles(128, 128) >= 128) {
     *name = "mmt4d_mfma_128x128";
-    return launch_tile<KIND, RHS_I4, G, 2, 2, 2>(m, stream);
+    if (direct) return launch_direct<KIND, RHS_I4, G, 2, 2, 4>(m, stream);
+    return launch_staged<KIND, RHS_I4, G, 2, 2, 2>(m, stream);
   }
   *name = "mmt4d_mfma_64x64";
-  return launch_tile<KIND, RHS_I4, G, 1, 1, 2>(m, stream);
+  if constexpr (!RHS_I4) {
+    if (direct) return launch_direct<KIND, RHS_I4, G, 1, 1, 8>(m, stream);
+  }
+  return launch_staged<KIND, RHS_I4, G, 1, 1, 2>(m, stream);
 }
 
 hipError_t launch_mfma(const Mmt4dArgs& a, hipStream_t stream, const char** name) {
