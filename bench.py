@@ -26,6 +26,15 @@ PEAK_INT8_TOPS = 5033.0     # dense int8 MFMA
 PEAK_F16_TFLOPS = 2516.0    # dense f16 / bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # HBM3E
 
+# HBM traffic of ONE launch of the headline kernel, measured with the
+# profiler's FETCH_SIZE and WRITE_SIZE counters (two separate counter runs of
+# this script, each reading scaled by what the same counter reports for a plain
+# device-to-device copy of known size: x2.00 for FETCH_SIZE, x1.00 for
+# WRITE_SIZE on this part). The algorithmic minimum is 32 MiB read + 64 MiB
+# written = 100.7 MB; reads above it are lhs/rhs panels fetched by more than
+# one of the 8 L2s. profiles/ holds the counter summaries.
+HEADLINE_TRAFFIC_BYTES = 168_128_922   # 49,326 KiB x 2.00 fetched + 65,536 KiB written
+
 
 def _mmt4d_params(abi, lhs, rhs, out, M, N, K, M0, N0, K0, flags):
     lb, rb, ob = abi.MMT4D_BITS[flags & 0xFF]
@@ -54,6 +63,21 @@ def _time_launches(torch, fn, steps, warmup):
     return e0.elapsed_time(e1) / steps, wall_ms / steps
 
 
+def _per_launch_ms(torch, fn, launches):
+    """Duration of each of `launches` calls of fn(), every one bracketed by its
+    own pair of HIP events: (median, min) in ms."""
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+             for _ in range(launches)]
+    torch.cuda.synchronize()
+    for e0, e1 in pairs:
+        e0.record()
+        fn()
+        e1.record()
+    torch.cuda.synchronize()
+    ms = sorted(e0.elapsed_time(e1) for e0, e1 in pairs)
+    return ms[len(ms) // 2], ms[0]
+
+
 def _headline(torch, lib, abi, synth, steps, warmup):
     import numpy as np
     M = N = 512
@@ -66,6 +90,7 @@ def _headline(torch, lib, abi, synth, steps, warmup):
     out = torch.empty(M * N * M0 * N0, dtype=torch.int32, device="cuda")
     p = _mmt4d_params(abi, lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), M, N, K, M0, N0, K0, flags)
     ev_ms, wall_ms = _time_launches(torch, lambda: lib.iree_uk_mmt4d_p(C.byref(p)), steps, warmup)
+    med_ms, min_ms = _per_launch_ms(torch, lambda: lib.iree_uk_mmt4d_p(C.byref(p)), max(steps, 20))
     kernel = lib.iree_uk_mi355x_last_kernel().decode()
     # Checksum of checksums, independent of any CPU code: the sum of all
     # outputs equals (column sums of A) . (column sums of B), with k running
@@ -74,7 +99,8 @@ def _headline(torch, lib, abi, synth, steps, warmup):
     b_cols = rhs.view(N, K, N0, K0).to(torch.int64).sum(dim=(0, 2)).reshape(-1)
     verified = bool((a_cols * b_cols).sum().item() == out.to(torch.int64).sum().item())
     ops = 2.0 * M * N * K * M0 * N0 * K0
-    return dict(ops=ops, ev_ms=ev_ms, wall_ms=wall_ms, kernel=kernel, verified=verified,
+    return dict(ops=ops, ev_ms=ev_ms, wall_ms=wall_ms, med_ms=med_ms, min_ms=min_ms, kernel=kernel,
+                verified=verified, params=p, keep=(lhs, rhs, out),
                 workload="iree_uk_mmt4d s8s8s32 logical 4096x4096x4096, tiles M0=N0=8 K0=4 "
                          "(lhs [512,1024,8,4], rhs [512,1024,8,4], out i32 [512,512,8,8]), "
                          "accumulate off, operands resident in HBM")
@@ -184,6 +210,16 @@ def _also(torch, lib, abi, synth, steps, warmup):
     timed_pair("pack_f32_8191x8190_transpose_inner_to_8191x512x16x1", pack_tr,
                (R * Cc + R * 512 * 16) * 4)
     del packed2
+    # The form the rhs of a matmul is packed in: both transposes, out [512, 8191, 16, 1]
+    # from the [8191, 8190] source read as its transpose.
+    packed3 = [torch.empty(512 * R * 16, dtype=torch.float32, device="cuda") for _ in range(2)]
+
+    def pack_rhs(i):
+        p = pack_params(i, abi.PACK_TRANSPOSE_INNER | abi.PACK_TRANSPOSE_OUTER, 512, R, 16, 1)
+        p.out_buffer = packed3[i].data_ptr()
+        return (lib.iree_uk_pack_p, p)
+    timed_pair("pack_f32_8191x8190_transpose_both_to_512x8191x16x1", pack_rhs, (R * Cc + 512 * R * 16) * 4)
+    del packed3
 
     def unpack_params(i):
         p = abi.UnpackParams()
@@ -289,6 +325,19 @@ def main():
     head = _headline(torch, lib, abi, synth, args.steps, args.warmup)
     also = None if args.no_also else _also(torch, lib, abi, synth, max(6, args.steps // 5), 2)
     lib.iree_uk_mi355x_set_stream(None, 0)
+    if also is not None:
+        # The same call the way the reference's callers make it: host pointers,
+        # synchronous (staged through device memory, PCIe-bound). Never `value`.
+        import numpy as np
+        lhs_h, rhs_h, out_d = (t.cpu().numpy() for t in head["keep"])
+        out_h = np.empty_like(out_d)
+        hp = _mmt4d_params(abi, lhs_h.ctypes.data, rhs_h.ctypes.data, out_h.ctypes.data, 512, 512, 1024, 8, 8, 4,
+                           abi.MMT4D_TYPE_S8S8S32)
+        lib.iree_uk_mmt4d_p(C.byref(hp))
+        t0 = time.perf_counter()
+        lib.iree_uk_mmt4d_p(C.byref(hp))
+        also["mmt4d_s8s8s32_4096_host_pointers_synchronous"] = {
+            "ms": round((time.perf_counter() - t0) * 1e3, 3), "bit_exact_vs_device_run": bool((out_h == out_d).all())}
     if args.calibrate_copy:
         a = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device="cuda").fill_(1)
         b = torch.empty_like(a)
@@ -312,8 +361,10 @@ def main():
         "config": {"workload": head["workload"], "kernel": head["kernel"],
                    "checksum_verified": head["verified"]},
         "roofline": {"bound": "mfma", "achieved": round(tops, 2), "peak": PEAK_INT8_TOPS,
-                     "unit": "TOP/s", "frac": round(tops / PEAK_INT8_TOPS, 4), "traffic": None,
-                     "kernel_ms": round(head["ev_ms"], 5)},
+                     "unit": "TOP/s", "frac": round(tops / PEAK_INT8_TOPS, 4),
+                     "traffic": HEADLINE_TRAFFIC_BYTES,
+                     "kernel_ms": round(head["ev_ms"], 5),
+                     "kernel_ms_median": round(head["med_ms"], 5), "kernel_ms_min": round(head["min_ms"], 5)},
         "cpu_baseline": cpu,
     }
     if cpu_arch is not None:
