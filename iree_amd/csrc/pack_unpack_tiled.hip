@@ -147,7 +147,15 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
         const int64_t row = row_base + r, col = col_base + (int64_t)cv * EPV;
         const uint8_t* g = a.src + (row * a.flat_stride0 + col) * E;
         if (row < a.size0 && col + EPV <= a.size1) {
-          regs[u].vec = *(const flat_vec_t*)g;
+          // Every byte is read once: streaming (non-temporal) accesses on both
+          // sides leave the caches to the other side's partial lines.
+          if constexpr (W == 16) {
+            typedef int v4a4 __attribute__((ext_vector_type(4), aligned(4)));
+            const v4a4 t = __builtin_nontemporal_load((const v4a4*)g);
+            regs[u].vec = Dwords4{(uint32_t)t.x, (uint32_t)t.y, (uint32_t)t.z, (uint32_t)t.w};
+          } else {
+            regs[u].vec = *(const flat_vec_t*)g;
+          }
         } else {
           // Edge: element by element, padding where the input ends.
 #pragma unroll
@@ -208,7 +216,10 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
       const int32_t e = (tid + 256 * u) * VE;
       first[u] = tiled_coord(a, e, tile0_base, tile1_base);
       if constexpr (UNPACK) {
-        if (first[u].in_range) regs[u].vec = *(const uint4*)(a.src + first[u].global_elem * E);
+        if (first[u].in_range) {
+          typedef int v4 __attribute__((ext_vector_type(4)));
+          regs[u].vec = __builtin_bit_cast(uint4, __builtin_nontemporal_load((const v4*)(a.src + first[u].global_elem * E)));
+        }
       }
     }
 #pragma unroll
@@ -226,7 +237,11 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
         piece_t* l = (piece_t*)(lds + row * a.pitch_bytes + col * E);
         if constexpr (UNPACK) *l = regs[u].piece[q]; else regs[u].piece[q] = *l;
       }
-      if constexpr (!UNPACK) *(uint4*)(a.dst + first[u].global_elem * E) = regs[u].vec;
+      if constexpr (!UNPACK) {
+        // Whole tiles, written once, never read back here: streaming store.
+        typedef int v4 __attribute__((ext_vector_type(4)));
+        __builtin_nontemporal_store(__builtin_bit_cast(v4, regs[u].vec), (v4*)(a.dst + first[u].global_elem * E));
+      }
     }
   };
 
