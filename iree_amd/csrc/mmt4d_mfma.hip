@@ -1,748 +1,10 @@
-// MFMA mmt4d for gfx950: s8s8s32, s8s4s32, f16f16f32 and bf16bf16f32.
-//
-// One workgroup of 256 threads (4 wavefronts in a 2x2 arrangement) computes a
-// block of (64*AM) lhs rows x (64*BN) rhs rows of the logical matrix; each
-// wavefront owns a (32*AM) x (32*BN) sub-block as AM x BN accumulator
-// fragments of one 32x32 MFMA each (v_mfma_i32_32x32x32_i8,
-// v_mfma_f32_32x32x16_f16/bf16: a single wavefront per SIMD keeps the matrix
-// pipe busy with these, which it cannot with the 16x16 shapes). The K dimension
-// is walked in chunks of 64 BYTES per operand row (64 int8 or 32 f16/bf16
-// values = two MFMA K-steps).
-//
-// Two kernels share this tiling and the epilogue:
-//   mmt4d_mfma_direct_kernel (the fast path): operands go global memory ->
-//     LDS directly, 16 contiguous bytes per lane, through a ring of LDS stages
-//     filled several chunks ahead; needs K to end on a chunk boundary and
-//     16-byte aligned operand rows.
-//   mmt4d_mfma_kernel (everything else the plan admits: ragged K, 4-byte
-//     aligned operands, narrow tiles): global -> registers (issued two chunks
-//     ahead) -> LDS -> registers (read one chunk ahead) -> MFMA.
-// In both, LDS holds the operands fragment-major, so that a wavefront fetches
-// a 32-row x 32-byte MFMA operand with conflict-free reads that are linear in
-// the lane number.
-//
-// Operand layouts. An mmt4d operand row (one i0 of one tile) is not contiguous
-// in memory: its K0 values of consecutive k are M0*K0 elements apart
-// (mmt4d_tile_generic.c:70-71). With RB = bytes of one (k, i0) row piece:
-//   RB multiple of 16: a lane's 16 operand bytes are contiguous in memory;
-//   RB == 4 (the 8x8x4 int8 tiles): a lane's 16 bytes come from 4 different k
-//     steps. K is permuted inside a chunk, identically for lhs and rhs, which
-//     leaves every integer sum unchanged (and reorders a float sum).
-// The int4 rhs of s8s4s32 is widened in registers: nibble n becomes the int8
-// value 16*n (sign in bit 7, no sign-extension step), the accumulators
-// therefore hold 16x the result and are shifted right by 4 at the end, which
-// is exact while 16*128*8*depth < 2^31.
-//
-// The MFMA is issued with the rhs fragment as its row operand and the lhs
-// fragment as its column operand, so a lane ends up with 4 consecutive j0 of
-// one output row: one 128-bit store per fragment into the [M0][N0] tile.
-#include "uk_internal.h"
+// Host side of the MFMA mmt4d kernels: which problems they cover, and the
+// dispatch to the per-type translation units (mmt4d_mfma_kernels.h describes
+// the kernels).
+#include "mmt4d_mfma_kernels.h"
 
 namespace uk {
 namespace {
-
-typedef int v4i32 __attribute__((ext_vector_type(4)));
-typedef int v16i32 __attribute__((ext_vector_type(16)));
-typedef float v16f32 __attribute__((ext_vector_type(16)));
-typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
-typedef __bf16 v8bf16 __attribute__((ext_vector_type(8)));
-
-enum Kind { kI8 = 0, kF16 = 1, kBF16 = 2 };
-
-struct MfmaArgs {
-  const uint8_t* lhs;
-  const uint8_t* rhs;
-  uint8_t* out;
-  int64_t lhs_stride_bytes;  // between consecutive lhs tiles rows (i)
-  int64_t rhs_stride_bytes;
-  int64_t out_stride0;       // elements
-  int32_t M, N, K;           // tile counts
-  int32_t log2_M0, log2_N0;
-  int32_t lhs_rb, rhs_rb;    // bytes of one (k, i0) row piece
-  int32_t log2_lhs_rb, log2_rhs_rb;
-  int32_t chunks;            // ceil(K * lhs_rb / 64)
-  int32_t tile_rows, tile_cols;  // grid of block tiles
-  int32_t accumulate;
-};
-
-template <int KIND>
-struct AccType { typedef v16i32 type; typedef int scalar; };
-template <> struct AccType<kF16> { typedef v16f32 type; typedef float scalar; };
-template <> struct AccType<kBF16> { typedef v16f32 type; typedef float scalar; };
-
-template <int KIND>
-__device__ __forceinline__ typename AccType<KIND>::type mfma(uint4 row_operand, uint4 col_operand,
-                                                             typename AccType<KIND>::type acc) {
-  if constexpr (KIND == kI8) {
-    return __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(v4i32, row_operand),
-                                                 __builtin_bit_cast(v4i32, col_operand), acc, 0, 0, 0);
-  } else if constexpr (KIND == kF16) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8f16, row_operand),
-                                                  __builtin_bit_cast(v8f16, col_operand), acc, 0, 0, 0);
-  } else {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf16, row_operand),
-                                                   __builtin_bit_cast(v8bf16, col_operand), acc, 0, 0, 0);
-  }
-}
-
-// 16 int4 values (two dwords, element 2b in the low nibble of byte b) to 16
-// int8 values equal to 16x the signed nibbles, in element order: the even and
-// the odd elements of a dword are isolated in the high nibbles of two dwords,
-// whose bytes are then interleaved.
-__device__ __forceinline__ uint4 widen_i4_times16(uint2 w) {
-  const uint32_t even0 = (w.x << 4) & 0xF0F0F0F0u, odd0 = w.x & 0xF0F0F0F0u;
-  const uint32_t even1 = (w.y << 4) & 0xF0F0F0F0u, odd1 = w.y & 0xF0F0F0F0u;
-  uint4 r;
-  r.x = __builtin_amdgcn_perm(odd0, even0, 0x05010400u);
-  r.y = __builtin_amdgcn_perm(odd0, even0, 0x07030602u);
-  r.z = __builtin_amdgcn_perm(odd1, even1, 0x05010400u);
-  r.w = __builtin_amdgcn_perm(odd1, even1, 0x07030602u);
-  return r;
-}
-
-// k step (relative to its chunk's first) that the 16-byte column `c` of an
-// operand row starts at.
-template <int G, bool I4>
-__device__ __forceinline__ int32_t piece_kstep(int c, int32_t log2_rb) {
-  if constexpr (I4) return (8 * c) >> log2_rb;
-  if constexpr (G == 16) return (16 * c) >> log2_rb;
-  return 4 * c;
-}
-
-// One 16-byte operand piece for LDS. `p` points at the piece's first byte for
-// the current chunk. G is the contiguous run in memory: 16 (one vector load),
-// 4 (gather one dword from each of 4 consecutive k steps, `kstep` bytes apart)
-// or, for I4, 8 bytes of nibbles widened to 16. With CHECKED, parts whose k
-// step `k1 (+d)` is not below K read as zero.
-template <int G, bool I4, bool CHECKED>
-__device__ __forceinline__ uint4 load_piece(const uint8_t* p, int64_t kstep, int32_t k1, int32_t K) {
-  uint4 v = make_uint4(0, 0, 0, 0);
-  if constexpr (I4) {
-    if (!CHECKED || k1 < K) v = widen_i4_times16(*(const uint2*)p);
-  } else if constexpr (G == 16) {
-    if (!CHECKED || k1 < K) v = *(const uint4*)p;
-  } else {
-    if (!CHECKED || k1 + 0 < K) v.x = *(const uint32_t*)(p);
-    if (!CHECKED || k1 + 1 < K) v.y = *(const uint32_t*)(p + kstep);
-    if (!CHECKED || k1 + 2 < K) v.z = *(const uint32_t*)(p + 2 * kstep);
-    if (!CHECKED || k1 + 3 < K) v.w = *(const uint32_t*)(p + 3 * kstep);
-  }
-  return v;
-}
-
-// Workgroup -> block tile. Consecutive workgroup ids go to different XCDs (8 of
-// them, each with its own L2), so ids are first regrouped so that one XCD works
-// on a contiguous range of tiles, then that range is walked in bands of 4 tile
-// rows so that neighbours share lhs and rhs panels. False: nothing to do.
-__device__ __forceinline__ bool locate_block(const MfmaArgs& a, int* tile_row, int* tile_col) {
-  const int total_tiles = a.tile_rows * a.tile_cols;
-  const int per_xcd = (total_tiles + 7) >> 3;
-  const int linear = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (linear >= total_tiles) return false;
-  constexpr int BAND = 4;
-  const int band = linear / (BAND * a.tile_cols);
-  const int band_first = band * BAND;
-  const int band_rows = min(a.tile_rows - band_first, BAND);
-  const int in_band = linear - band * BAND * a.tile_cols;
-  *tile_row = band_first + in_band % band_rows;
-  *tile_col = in_band / band_rows;
-  return true;
-}
-
-// Writes one wavefront's accumulators. Lane l holds, for fragment (i, j): lhs
-// row 32*i + (l & 31) and, in accumulator registers 4*q .. 4*q+3, rhs rows
-// 32*j + 8*q + 4*(l >> 5) + {0..3} of the wavefront's sub-block, which starts at
-// (wave_row, wave_col) of the logical matrix: four consecutive j0 of one output
-// row, one 128-bit store. When accumulating, all of a row's loads are issued
-// before the first add, so their latencies overlap.
-template <int KIND, bool RHS_I4, int AM, int BN>
-__device__ __forceinline__ void store_block(const MfmaArgs& a, typename AccType<KIND>::type (&acc)[AM][BN],
-                                            int64_t wave_row, int64_t wave_col, int lane) {
-  typedef typename AccType<KIND>::scalar scalar_t;
-  typedef scalar_t quad_t __attribute__((ext_vector_type(4)));
-  const int32_t M0 = 1 << a.log2_M0, N0 = 1 << a.log2_N0;
-  const int64_t total_rows = (int64_t)a.M << a.log2_M0;
-  const int64_t total_cols = (int64_t)a.N << a.log2_N0;
-  const int64_t row0 = wave_row + (lane & 31);
-  const int64_t col0 = wave_col + 4 * (lane >> 5);
-  // Byte offset of quad (j, q) from the sub-block's first column tile (the same
-  // for every row, and small) and whether the quad lies inside the matrix.
-  const int64_t first_col_tile = wave_col >> a.log2_N0;
-  uint8_t* wave_out = a.out + 4 * (first_col_tile << (a.log2_M0 + a.log2_N0));
-  uint32_t col_off[BN][4];
-  uint32_t col_inside = 0;
-#pragma unroll
-  for (int j = 0; j < BN; ++j)
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int64_t col = col0 + 32 * j + 8 * q;
-      col_off[j][q] =
-          (uint32_t)(4 * ((((col >> a.log2_N0) - first_col_tile) << (a.log2_M0 + a.log2_N0)) + (col & (N0 - 1))));
-      if (col < total_cols) col_inside |= 1u << (4 * j + q);
-    }
-#pragma unroll
-  for (int i = 0; i < AM; ++i) {
-    const int64_t row = min(row0 + 32 * i, total_rows - 1);
-    const bool row_inside = row0 + 32 * i < total_rows;
-    uint8_t* row_out = wave_out + 4 * ((row >> a.log2_M0) * a.out_stride0 + ((row & (M0 - 1)) << a.log2_N0));
-#pragma unroll
-    for (int j = 0; j < BN; ++j) {
-      // Pin the fragment where it is until its turn: left alone, the compiler
-      // moves all 256 accumulators to ordinary registers right after the main
-      // loop, and there are not that many.
-      typename AccType<KIND>::type frag = acc[i][j];
-      asm volatile("" : "+a"(frag));
-      quad_t v[4];
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        v[q] = quad_t{frag[4 * q], frag[4 * q + 1], frag[4 * q + 2], frag[4 * q + 3]};
-        if constexpr (RHS_I4) v[q] = v[q] >> 4;
-      }
-      if (a.accumulate) {
-        quad_t old[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          old[q] = quad_t{0, 0, 0, 0};
-          if (row_inside && (col_inside >> (4 * j + q) & 1)) old[q] = *(const quad_t*)(row_out + col_off[j][q]);
-        }
-#pragma unroll
-        for (int q = 0; q < 4; ++q) v[q] += old[q];
-      }
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-        if (row_inside && (col_inside >> (4 * j + q) & 1)) *(quad_t*)(row_out + col_off[j][q]) = v[q];
-      // Keep the fragments apart: hoisting all address arithmetic and
-      // accumulator reads to the top costs more registers than there are.
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  }
-}
-
-template <int KIND, bool RHS_I4, int G, int AM, int BN, int MIN_BLOCKS, bool TAIL>
-__global__ __launch_bounds__(256, MIN_BLOCKS) void mmt4d_mfma_kernel(const MfmaArgs a) {
-  typedef typename AccType<KIND>::type acc_t;
-  constexpr int BLOCK_ROWS = 64 * AM;  // lhs rows per workgroup
-  constexpr int BLOCK_COLS = 64 * BN;  // rhs rows per workgroup
-  constexpr int A_PIECES = BLOCK_ROWS * 4;  // 16-byte pieces per chunk
-  constexpr int B_PIECES = BLOCK_COLS * 4;
-  constexpr int A_PER_THREAD = (A_PIECES + 255) / 256;
-  constexpr int B_PER_THREAD = (B_PIECES + 255) / 256;
-  static_assert(A_PIECES % 256 == 0 && B_PIECES % 256 == 0, "block tile too small");
-  __shared__ uint4 lds_a[2][A_PIECES];
-  __shared__ uint4 lds_b[2][B_PIECES];
-
-  int tile_row, tile_col;
-  if (!locate_block(a, &tile_row, &tile_col)) return;
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wave_m = wave >> 1, wave_n = wave & 1;
-
-  const int32_t M0 = 1 << a.log2_M0, N0 = 1 << a.log2_N0;
-  const int64_t total_rows = (int64_t)a.M << a.log2_M0;
-  const int64_t total_cols = (int64_t)a.N << a.log2_N0;
-  const int64_t lhs_kstep = (int64_t)a.lhs_rb << a.log2_M0;
-  const int64_t rhs_kstep = (int64_t)a.rhs_rb << a.log2_N0;
-  // k steps covered by one chunk (64 bytes of an lhs row).
-  const int32_t ksteps_per_chunk = 64 >> a.log2_lhs_rb;
-
-  // Workgroup-uniform bases and 32-bit per-piece offsets from them. Piece
-  // p = tid + 256*s lands at LDS slot p: fragment (p >> 7), 16-byte column
-  // (p >> 5) & 3, row p & 31 of the fragment (column c is K-step c >> 1, lane
-  // half c & 1 of the MFMA operand). Rows past the end of the matrix
-  // are redirected to its last row: their products are computed, never stored.
-  const int64_t first_row = (int64_t)tile_row * BLOCK_ROWS;
-  const int64_t first_col = (int64_t)tile_col * BLOCK_COLS;
-  const uint8_t* lhs_base = a.lhs + (first_row >> a.log2_M0) * a.lhs_stride_bytes;
-  const uint8_t* rhs_base = a.rhs + (first_col >> a.log2_N0) * a.rhs_stride_bytes;
-  uint32_t a_off[A_PER_THREAD], b_off[B_PER_THREAD];
-#pragma unroll
-  for (int s = 0; s < A_PER_THREAD; ++s) {
-    const int p = tid + 256 * s;
-    const int c = (p >> 5) & 3;
-    const int64_t row = min(first_row + (p >> 7) * 32 + (p & 31), total_rows - 1);
-    const int64_t tile = (row >> a.log2_M0) - (first_row >> a.log2_M0);
-    const int32_t col_byte = G == 16 ? 16 * c : 0;
-    const int32_t k1 = piece_kstep<G, false>(c, a.log2_lhs_rb);
-    a_off[s] = (uint32_t)(tile * a.lhs_stride_bytes + (row & (M0 - 1)) * a.lhs_rb +
-                          k1 * lhs_kstep + (col_byte & (a.lhs_rb - 1)));
-  }
-#pragma unroll
-  for (int s = 0; s < B_PER_THREAD; ++s) {
-    const int p = tid + 256 * s;
-    const int c = (p >> 5) & 3;
-    const int64_t row = min(first_col + (p >> 7) * 32 + (p & 31), total_cols - 1);
-    const int64_t tile = (row >> a.log2_N0) - (first_col >> a.log2_N0);
-    const int32_t col_byte = RHS_I4 ? 8 * c : (G == 16 ? 16 * c : 0);
-    const int32_t k1 = piece_kstep<G, RHS_I4>(c, a.log2_rhs_rb);
-    b_off[s] = (uint32_t)(tile * a.rhs_stride_bytes + (row & (N0 - 1)) * a.rhs_rb +
-                          k1 * rhs_kstep + (col_byte & (a.rhs_rb - 1)));
-  }
-
-  acc_t acc[AM][BN];
-#pragma unroll
-  for (int i = 0; i < AM; ++i)
-#pragma unroll
-    for (int j = 0; j < BN; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
-
-  // Global -> register prefetch of one chunk, two chunks deep: while chunk kc
-  // is multiplied, chunk kc + 1 moves from registers to LDS and chunks kc + 2
-  // and kc + 3 are in flight from memory (a load takes longer than one chunk
-  // of MFMAs, so a single chunk of lookahead would stall every iteration).
-  uint4 a_pre[2][A_PER_THREAD], b_pre[2][B_PER_THREAD];
-  auto fetch = [&](int kc, uint4* a_next, uint4* b_next) {
-    const int32_t k1_0 = kc * ksteps_per_chunk;
-    const uint8_t* la = lhs_base + (int64_t)k1_0 * lhs_kstep;
-    const uint8_t* lb = rhs_base + (int64_t)k1_0 * rhs_kstep;
-#pragma unroll
-    for (int s = 0; s < A_PER_THREAD; ++s)
-      a_next[s] = load_piece<G, false, false>(la + a_off[s], lhs_kstep, 0, 0);
-#pragma unroll
-    for (int s = 0; s < B_PER_THREAD; ++s)
-      b_next[s] = load_piece<G, RHS_I4, false>(lb + b_off[s], rhs_kstep, 0, 0);
-  };
-  // Same for a chunk that K ends inside of: missing k steps read as zero.
-  auto fetch_checked = [&](int kc, uint4* a_next, uint4* b_next) {
-    const int32_t k1_0 = kc * ksteps_per_chunk;
-    const uint8_t* la = lhs_base + (int64_t)k1_0 * lhs_kstep;
-    const uint8_t* lb = rhs_base + (int64_t)k1_0 * rhs_kstep;
-#pragma unroll
-    for (int s = 0; s < A_PER_THREAD; ++s)
-      a_next[s] = load_piece<G, false, true>(
-          la + a_off[s], lhs_kstep,
-          k1_0 + piece_kstep<G, false>(((tid + 256 * s) >> 5) & 3, a.log2_lhs_rb), a.K);
-#pragma unroll
-    for (int s = 0; s < B_PER_THREAD; ++s)
-      b_next[s] = load_piece<G, RHS_I4, true>(
-          lb + b_off[s], rhs_kstep,
-          k1_0 + piece_kstep<G, RHS_I4>(((tid + 256 * s) >> 5) & 3, a.log2_rhs_rb), a.K);
-  };
-  auto stash = [&](int stage, const uint4* a_next, const uint4* b_next) {
-#pragma unroll
-    for (int s = 0; s < A_PER_THREAD; ++s) lds_a[stage][tid + 256 * s] = a_next[s];
-#pragma unroll
-    for (int s = 0; s < B_PER_THREAD; ++s) lds_b[stage][tid + 256 * s] = b_next[s];
-  };
-
-  // Fragment registers, double buffered: while the MFMAs of chunk kc run from
-  // one set, the fragments of chunk kc + 1 are read from LDS into the other.
-  // The loop is unrolled by two so the sets swap roles without copies, and its
-  // body is branch-free (the prefetch index is clamped instead) so that LDS
-  // reads, global loads and MFMAs can be scheduled against each other.
-  uint4 pa[AM][2], pb[BN][2], qa[AM][2], qb[BN][2];
-  auto read_frags = [&](int stage, uint4 (*fa)[2], uint4 (*fb)[2]) {
-    const uint4* frag_a = &lds_a[stage][(wave_m * AM) * 128 + lane];
-    const uint4* frag_b = &lds_b[stage][(wave_n * BN) * 128 + lane];
-    // K-step 0 first: it is what the next step's first MFMAs consume.
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-#pragma unroll
-      for (int j = 0; j < BN; ++j) fb[j][kk] = frag_b[j * 128 + kk * 64];
-#pragma unroll
-      for (int i = 0; i < AM; ++i) fa[i][kk] = frag_a[i * 128 + kk * 64];
-    }
-  };
-  auto multiply = [&](const uint4 (*fa)[2], const uint4 (*fb)[2], int kk) {
-#pragma unroll
-    for (int i = 0; i < AM; ++i)
-#pragma unroll
-      for (int j = 0; j < BN; ++j) acc[i][j] = mfma<KIND>(fb[j][kk], fa[i][kk], acc[i][j]);
-  };
-  // Chunks that lie entirely inside K run through the pipeline; a trailing
-  // partial chunk is handled after it, unpipelined.
-  const int full_chunks = a.K / ksteps_per_chunk;
-  const int last_chunk = full_chunks - 1;
-  // One pipeline step for chunk kc, whose fragments are in `cur`:
-  //   registers(kc + 1) -> LDS stage, first half of the MFMAs (covers the LDS
-  //   write latency), barrier, global loads of chunk kc + 3 into the register
-  //   set just freed, LDS reads of the fragments of chunk kc + 1, second half
-  //   of the MFMAs (covers the LDS read latency). Prefetch indices are clamped
-  //   to the last full chunk, so the body is branch-free.
-  auto step = [&](int kc, int stage, const uint4 (*cur_a)[2], const uint4 (*cur_b)[2],
-                  uint4 (*nxt_a)[2], uint4 (*nxt_b)[2]) {
-    // A wavefront issues in order, so memory instructions only overlap with
-    // the matrix pipe if they sit between MFMAs in program order: the two
-    // halves below are interleaved one MFMA at a time with the LDS writes and
-    // global loads (first half) and with the LDS reads (second half).
-    constexpr int MFMAS = AM * BN;  // per half
-    constexpr int WRITES = A_PER_THREAD + B_PER_THREAD;
-    constexpr int LOADS = (G == 4 ? 4 : 1) * A_PER_THREAD + ((G == 4 && !RHS_I4) ? 4 : 1) * B_PER_THREAD;
-    constexpr int READS = 2 * (AM + BN);
-    stash(stage, a_pre[stage], b_pre[stage]);
-    fetch(min(kc + 3, last_chunk), a_pre[stage], b_pre[stage]);
-    multiply(cur_a, cur_b, 0);
-#pragma unroll
-    for (int m = 0; m < MFMAS; ++m) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
-      if (m < WRITES) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // one LDS write
-      constexpr int LOADS_PER = (LOADS + MFMAS - 1) / MFMAS;
-      if (m * LOADS_PER < LOADS) {
-        __builtin_amdgcn_sched_group_barrier(0x002, 2 * LOADS_PER, 0);  // address arithmetic
-        __builtin_amdgcn_sched_group_barrier(0x020, LOADS_PER, 0);      // global loads
-      }
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    __syncthreads();
-    read_frags(stage, nxt_a, nxt_b);
-    multiply(cur_a, cur_b, 1);
-#pragma unroll
-    for (int m = 0; m < MFMAS; ++m) {
-      constexpr int READS_PER = (READS + MFMAS - 1) / MFMAS;
-      if (m * READS_PER < READS) __builtin_amdgcn_sched_group_barrier(0x100, READS_PER, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-  };
-
-  if (full_chunks > 0) {
-    // Chunk c travels through register set c & 1 and LDS stage c & 1.
-    fetch(0, a_pre[0], b_pre[0]);
-    fetch(min(1, last_chunk), a_pre[1], b_pre[1]);
-    stash(0, a_pre[0], b_pre[0]);
-    fetch(min(2, last_chunk), a_pre[0], b_pre[0]);
-    __syncthreads();
-    read_frags(0, pa, pb);
-    int kc = 0;
-    for (; kc + 1 < full_chunks; kc += 2) {
-      step(kc, 1, pa, pb, qa, qb);
-      step(kc + 1, 0, qa, qb, pa, pb);
-    }
-    if (kc < full_chunks) {
-      multiply(pa, pb, 0);
-      multiply(pa, pb, 1);
-    }
-  }
-  if constexpr (TAIL) {
-    fetch_checked(full_chunks, a_pre[0], b_pre[0]);
-    __syncthreads();  // every wavefront is done reading LDS stage 0
-    stash(0, a_pre[0], b_pre[0]);
-    __syncthreads();
-    read_frags(0, pa, pb);
-    multiply(pa, pb, 0);
-    multiply(pa, pb, 1);
-  }
-
-  store_block<KIND, RHS_I4, AM, BN>(a, acc, first_row + wave_m * (32 * AM), first_col + wave_n * (32 * BN),
-                                    lane);
-}
-
-// ---------------------------------------------------------------------------
-// Direct-to-LDS variant: the same block tiling, but operand pieces travel
-// global memory -> LDS without passing through registers
-// (global_load_lds_dwordx4: lane l of a wavefront writes its 16 bytes at
-// M0 + 16*l), through a ring of 4 LDS stages filled three chunks ahead of the
-// MFMAs. It needs no register prefetch buffers, no LDS writes and no
-// data-dependent waits other than one counter wait per chunk. It covers the
-// int8/f16/bf16 rhs (no nibble widening on the way) and K that ends on a chunk
-// boundary; everything else uses the kernel above.
-//
-// Every load moves 16 contiguous bytes per lane, also for the 4-byte row
-// pieces of e.g. the 8x8x4 int8 tiles (G == 4), where 16 contiguous bytes are
-// 4 consecutive rows of one k step: there the transposition to "one row, 16
-// bytes of K" happens on the way out of LDS, with four 32-bit reads per
-// fragment instead of one 128-bit read, and the loads are arranged so that
-// those reads are linear in the lane number (conflict-free).
-//
-// The loads are issued from inline assembly: the compiler cannot see that they
-// write LDS, so it does not serialise the LDS reads against them; ordering is
-// enforced by hand with s_waitcnt vmcnt + a workgroup barrier once per chunk.
-extern __shared__ uint4 ring[];
-
-// One wavefront-wide load of 64 x 16 bytes to LDS byte offset `lds_off`
-// (wavefront-uniform) from `base` (uniform) + per-lane byte offset `voff`.
-__device__ __forceinline__ void load_to_lds(uint32_t lds_off, uint32_t voff, const uint8_t* base) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-               :
-               : "s"(lds_off), "v"(voff), "s"(base)
-               : "memory");
-}
-
-template <int N>
-__device__ __forceinline__ void wait_loads_but() {
-  static_assert(N >= 0 && N <= 63, "vmcnt is a 6-bit counter");
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-
-template <int KIND, bool RHS_I4, int G, int AM, int BN, int STAGES>
-__global__ __launch_bounds__(256) void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
-  typedef typename AccType<KIND>::type acc_t;
-  static_assert(!RHS_I4 || (G == 16 && BN >= 2), "int4 rhs: 16-byte pieces, at least one fragment per wavefront");
-  constexpr int BLOCK_ROWS = 64 * AM, BLOCK_COLS = 64 * BN;
-  // 16-byte pieces per chunk: 64 bytes of K per row, 32 bytes for an int4 rhs.
-  constexpr int A_PIECES = BLOCK_ROWS * 4, B_PIECES = BLOCK_COLS * (RHS_I4 ? 2 : 4);
-  // Stage size rounded up to a power of two so that ring offsets wrap with a mask.
-  constexpr int STAGE_PIECES = A_PIECES + B_PIECES <= 512    ? 512
-                               : A_PIECES + B_PIECES <= 1024 ? 1024
-                                                             : 2048;
-  static_assert(A_PIECES + B_PIECES <= STAGE_PIECES, "stage too small");
-  constexpr int AHEAD = STAGES - 1;  // chunks in flight ahead of the one being multiplied
-  static_assert(STAGES >= 4 && (STAGES & (STAGES - 1)) == 0, "ring depth");
-  // Load instructions per wavefront and chunk (64 lanes x 16 bytes each), each
-  // with its own per-lane offset.
-  constexpr int A_LOADS = A_PIECES / 256, B_LOADS = B_PIECES / 256;
-  constexpr int LOADS = A_LOADS + B_LOADS;
-  static_assert(A_PIECES % 256 == 0 && B_PIECES % 256 == 0, "block tile too small");
-  static_assert((AHEAD - 1) * LOADS <= 63, "the loads in flight must fit the 6-bit counter");
-
-  int tile_row, tile_col;
-  if (!locate_block(a, &tile_row, &tile_col)) return;
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wave_m = wave >> 1, wave_n = wave & 1;
-
-  const int32_t M0 = 1 << a.log2_M0, N0 = 1 << a.log2_N0;
-  const int64_t total_rows = (int64_t)a.M << a.log2_M0;
-  const int64_t total_cols = (int64_t)a.N << a.log2_N0;
-  const int64_t lhs_kstep = (int64_t)a.lhs_rb << a.log2_M0;
-  const int64_t rhs_kstep = (int64_t)a.rhs_rb << a.log2_N0;
-  const int32_t ksteps_per_chunk = 64 >> a.log2_lhs_rb;
-  const int64_t lhs_chunk_bytes = ksteps_per_chunk * lhs_kstep;
-  const int64_t rhs_chunk_bytes = ksteps_per_chunk * rhs_kstep;
-
-  const int64_t first_row = (int64_t)tile_row * BLOCK_ROWS;
-  const int64_t first_col = (int64_t)tile_col * BLOCK_COLS;
-  const uint8_t* lhs_base = a.lhs + (first_row >> a.log2_M0) * a.lhs_stride_bytes;
-  const uint8_t* rhs_base = a.rhs + (first_col >> a.log2_N0) * a.rhs_stride_bytes;
-
-  // Load t of wavefront w fills the 16-byte LDS slots 64*m .. 64*m + 63 of its
-  // operand, m = 4*t + w, lane l the slot 64*m + l.
-  //   G == 16: slot p holds fragment p >> 7, 16-byte column (p >> 5) & 3 (K-step
-  //     c >> 1, lane half c & 1 of the MFMA operand), row p & 31: a fragment is
-  //     read back with one 128-bit read at slot 128*f + 64*kk + lane.
-  //   G == 4: slot 64*m + l holds rows 4*g .. 4*g + 3 (g = l & 7) of fragment
-  //     m >> 1 at k step 8*(m & 1) + 4*h + d of the chunk (h = (l >> 3) & 1,
-  //     d = l >> 4). Dword 64*(8*f + 4*kk + d) + 32*h + r of the operand is then
-  //     row r of fragment f at that k step: the MFMA operand of lane 32*h + r
-  //     for K-step kk is dwords d = 0..3, each read linear in the lane number.
-  //     K is permuted inside a chunk, identically for lhs and rhs.
-  //   int4 rhs: slot 64*f + 32*h + r holds nibbles 32*h .. 32*h + 31 of row r of
-  //     fragment f: lane 32*h + r reads that slot once per chunk and widens its
-  //     first 8 bytes for K-step 0, its last 8 for K-step 1. The lhs columns are
-  //     assigned to match: (K-step kk, lane half h) gets 16-byte column kk + 2*h.
-  // Rows past the end of the matrix are redirected to its last row (group):
-  // their products are computed, never stored.
-  auto row_offset = [&](int64_t row, int64_t last, int64_t first, int log2_t0, int64_t stride_bytes,
-                        int32_t rb) -> int64_t {
-    row = min(row, last);
-    const int64_t tile = (row >> log2_t0) - (first >> log2_t0);
-    return tile * stride_bytes + (row & ((1 << log2_t0) - 1)) * rb;
-  };
-  uint32_t a_off[A_LOADS], b_off[B_LOADS];
-  if constexpr (G == 16) {
-#pragma unroll
-    for (int t = 0; t < A_LOADS; ++t) {
-      const int p = tid + 256 * t;
-      const int c = RHS_I4 ? ((p >> 6) & 1) + 2 * ((p >> 5) & 1) : (p >> 5) & 3;
-      a_off[t] = (uint32_t)(row_offset(first_row + (p >> 7) * 32 + (p & 31), total_rows - 1, first_row,
-                                       a.log2_M0, a.lhs_stride_bytes, a.lhs_rb) +
-                            ((16 * c) >> a.log2_lhs_rb) * lhs_kstep + ((16 * c) & (a.lhs_rb - 1)));
-    }
-#pragma unroll
-    for (int t = 0; t < B_LOADS; ++t) {
-      const int p = tid + 256 * t;
-      const int c = RHS_I4 ? (p >> 5) & 1 : (p >> 5) & 3;
-      const int row = RHS_I4 ? (p >> 6) * 32 + (p & 31) : (p >> 7) * 32 + (p & 31);
-      b_off[t] = (uint32_t)(row_offset(first_col + row, total_cols - 1, first_col, a.log2_N0,
-                                       a.rhs_stride_bytes, a.rhs_rb) +
-                            ((16 * c) >> a.log2_rhs_rb) * rhs_kstep + ((16 * c) & (a.rhs_rb - 1)));
-    }
-  } else {
-    const int g = lane & 7, k1 = 4 * ((lane >> 3) & 1) + (lane >> 4);
-#pragma unroll
-    for (int t = 0; t < A_LOADS; ++t)
-      a_off[t] = (uint32_t)(row_offset(first_row + 32 * (2 * t + (wave >> 1)) + 4 * g, total_rows - 4, first_row,
-                                       a.log2_M0, a.lhs_stride_bytes, a.lhs_rb) + k1 * lhs_kstep);
-#pragma unroll
-    for (int t = 0; t < B_LOADS; ++t)
-      b_off[t] = (uint32_t)(row_offset(first_col + 32 * (2 * t + (wave >> 1)) + 4 * g, total_cols - 4, first_col,
-                                       a.log2_N0, a.rhs_stride_bytes, a.rhs_rb) + k1 * rhs_kstep);
-  }
-  // G == 4: this wavefront's loads all belong to K-step wave & 1.
-  const int64_t lhs_wave_bytes = G == 4 ? 8 * (wave & 1) * lhs_kstep : 0;
-  const int64_t rhs_wave_bytes = G == 4 ? 8 * (wave & 1) * rhs_kstep : 0;
-
-  acc_t acc[AM][BN];
-#pragma unroll
-  for (int i = 0; i < AM; ++i)
-#pragma unroll
-    for (int j = 0; j < BN; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
-
-  const int chunks = a.chunks;  // all full
-  const int last_chunk = chunks - 1;
-
-  // Load number `n` (compile-time after unrolling) of the chunk whose operand
-  // bases are la / lb, into the stage at LDS byte offset `stage_off`.
-  auto issue_load = [&](int n, uint32_t stage_off, const uint8_t* la, const uint8_t* lb) {
-    const bool is_a = n < A_LOADS;
-    const int t = is_a ? n : n - A_LOADS;
-    load_to_lds(stage_off + (is_a ? 0 : A_PIECES * 16) + (256 * t + 64 * wave) * 16,
-                is_a ? a_off[t] : b_off[t], is_a ? la : lb);
-  };
-  auto issue_chunk = [&](int kc) {
-    const int idx = min(kc, last_chunk);
-    const uint32_t stage_off = (uint32_t)(kc & (STAGES - 1)) * (STAGE_PIECES * 16);
-    const uint8_t* la = lhs_base + idx * lhs_chunk_bytes + lhs_wave_bytes;
-    const uint8_t* lb = rhs_base + idx * rhs_chunk_bytes + rhs_wave_bytes;
-#pragma unroll
-    for (int n = 0; n < LOADS; ++n) issue_load(n, stage_off, la, lb);
-  };
-
-  uint4 pa[AM][2], pb[BN][2], qa[AM][2], qb[BN][2];
-  // Fragment f of an operand at 16-byte slot `operand` of the ring, K-step kk.
-  auto read_frag = [&](int operand, int f, int kk) -> uint4 {
-    if (RHS_I4 && operand >= A_PIECES) {
-      const uint4 raw = ring[operand + 64 * f + lane];
-      return widen_i4_times16(kk ? make_uint2(raw.z, raw.w) : make_uint2(raw.x, raw.y));
-    }
-    if constexpr (G == 16) {
-      return ring[operand + 128 * f + 64 * kk + lane];
-    } else {
-      const uint32_t* words = (const uint32_t*)(ring + operand) + 64 * (8 * f + 4 * kk) + lane;
-      return make_uint4(words[0], words[64], words[128], words[192]);
-    }
-  };
-  const int frag_a0 = wave_m * AM, frag_b0 = wave_n * BN;
-
-  // Loop-carried, wavefront-uniform state: where the next chunk to load comes
-  // from and goes to, and the stage the next fragments are read from. Kept as
-  // running values (a few scalar adds per step) rather than recomputed from the
-  // chunk number (64-bit multiplies on the scalar unit, in front of the step's
-  // first MFMA).
-  constexpr uint32_t STAGE_BYTES = STAGE_PIECES * 16, RING_BYTES = STAGES * STAGE_BYTES;
-  static_assert((RING_BYTES & (RING_BYTES - 1)) == 0, "ring offsets wrap with a mask");
-  const uint8_t* load_a = lhs_base + min(AHEAD, last_chunk) * lhs_chunk_bytes + lhs_wave_bytes;
-  const uint8_t* load_b = rhs_base + min(AHEAD, last_chunk) * rhs_chunk_bytes + rhs_wave_bytes;
-  int load_chunk = AHEAD;
-  uint32_t load_stage_off = AHEAD * STAGE_BYTES % RING_BYTES;
-  uint32_t read_stage_off = STAGE_BYTES;
-  const uint32_t frag_a_off = (uint32_t)((wave_m * AM) * 128) * 16;
-  const uint32_t frag_b_off = (uint32_t)(A_PIECES + (wave_n * BN) * (RHS_I4 ? 64 : 128)) * 16;
-  const uint8_t* ring_bytes = (const uint8_t*)ring + (G == 16 ? 16 : 4) * lane;
-
-  // One pipeline step for the chunk whose fragments are in `cur`:
-  //   a few MFMAs first (they only need registers, and keep the matrix pipe
-  //   fed across the barrier); wait until this wavefront's loads of the next
-  //   chunk have landed; barrier (now everyone's have, and everyone is done
-  //   reading the stage of the previous chunk); then the remaining MFMAs with,
-  //   between them, the loads of the chunk three ahead into the stage just
-  //   freed and the LDS reads of the next chunk's fragments.
-  // A wavefront issues in order and a memory instruction takes several cycles
-  // to issue, so more than one or two of them between two MFMAs lets the
-  // matrix pipe run dry: they are dealt out one (half) fragment and at most one
-  // load per MFMA. The reads end a quarter of the step before its end, so that
-  // the last of them has returned when the next step starts; fragments are
-  // read in the order the next step consumes them.
-  auto step = [&](const uint4 (*cur_a)[2], const uint4 (*cur_b)[2], uint4 (*nxt_a)[2], uint4 (*nxt_b)[2]) {
-    constexpr int MFMAS = 2 * AM * BN;
-    constexpr int PARTS = G == 4 ? 2 : 1;  // LDS read instructions per fragment (after pairing)
-    // Read units, in the order the next step consumes them: per K-step the rhs
-    // fragments, then the lhs fragments. An int4 rhs fragment is read once, raw,
-    // for both K-steps (first), and widened after the last read has been issued.
-    constexpr int B_UNITS = RHS_I4 ? BN : 0;
-    constexpr int READS = RHS_I4 ? BN + 2 * AM : 2 * (AM + BN) * PARTS;
-    constexpr int LEAD = MFMAS >= 16 ? 4 : (MFMAS >= 8 ? 2 : 0);   // MFMAs ahead of the barrier
-    constexpr int TAIL_FREE = MFMAS >= 8 ? MFMAS / 4 : 0;          // MFMAs after the last read
-    constexpr int SLOTS = MFMAS - LEAD - TAIL_FREE;                // MFMAs that carry memory work
-    static_assert(SLOTS >= 1, "no room for the memory instructions");
-    static_assert(!RHS_I4 || TAIL_FREE >= 1, "nowhere to widen");
-    auto multiply = [&](int m) {
-      const int kk = m / (AM * BN), i = (m % (AM * BN)) / BN, j = m % BN;
-      acc[i][j] = mfma<KIND>(cur_b[j][kk], cur_a[i][kk], acc[i][j]);
-    };
-#pragma unroll
-    for (int m = 0; m < LEAD; ++m) multiply(m);
-    __builtin_amdgcn_sched_barrier(0);
-    wait_loads_but<LOADS*(AHEAD - 2)>();
-    __builtin_amdgcn_s_barrier();
-    const uint8_t* read_a = ring_bytes + read_stage_off + frag_a_off;
-    const uint8_t* read_b = ring_bytes + read_stage_off + frag_b_off;
-    uint4 raw_b[RHS_I4 ? BN : 1];
-#pragma unroll
-    for (int m = LEAD; m < MFMAS; ++m) {
-      const int slot = m - LEAD;
-      if (slot < SLOTS) {
-#pragma unroll
-        for (int n = slot * LOADS / SLOTS; n < (slot + 1) * LOADS / SLOTS; ++n)
-          issue_load(n, load_stage_off, load_a, load_b);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int u = slot * READS / SLOTS; u < (slot + 1) * READS / SLOTS; ++u) {
-          if constexpr (RHS_I4) {
-            if (u < B_UNITS) {
-              raw_b[u] = *(const uint4*)(read_b + (64 * u) * 16);
-            } else {
-              const int kk = (u - B_UNITS) / AM, i = (u - B_UNITS) % AM;
-              nxt_a[i][kk] = *(const uint4*)(read_a + (128 * i + 64 * kk) * 16);
-            }
-          } else {
-            const int f = u / PARTS, part = u % PARTS;
-            const int kk = f / (AM + BN), e = f % (AM + BN);
-            uint4& dst = e < BN ? nxt_b[e][kk] : nxt_a[e - BN][kk];
-            const uint8_t* src = e < BN ? read_b : read_a;
-            const int frag = e < BN ? e : e - BN;
-            if constexpr (G == 16) {
-              dst = *(const uint4*)(src + (128 * frag + 64 * kk) * 16);
-            } else {
-              const uint32_t* words = (const uint32_t*)src + 64 * (8 * frag + 4 * kk + 2 * part);
-              if (part == 0) { dst.x = words[0]; dst.y = words[64]; }
-              else { dst.z = words[0]; dst.w = words[64]; }
-            }
-          }
-        }
-      } else if constexpr (RHS_I4) {
-        // Widening, dealt out over the MFMAs that carry no memory work.
-        const int tail = slot - SLOTS;
-#pragma unroll
-        for (int w = tail * 2 * BN / TAIL_FREE; w < (tail + 1) * 2 * BN / TAIL_FREE; ++w) {
-          const int kk = w / BN, j = w % BN;
-          nxt_b[j][kk] = widen_i4_times16(kk ? make_uint2(raw_b[j].z, raw_b[j].w) : make_uint2(raw_b[j].x, raw_b[j].y));
-        }
-      }
-      multiply(m);
-      if (m == MFMAS - 1) {
-        // Advance the running state (clamped at the last chunk: the loads
-        // issued beyond it are redundant, their stages are never read).
-        const bool more = load_chunk < last_chunk;
-        load_a += more ? lhs_chunk_bytes : 0;
-        load_b += more ? rhs_chunk_bytes : 0;
-        ++load_chunk;
-        load_stage_off = (load_stage_off + STAGE_BYTES) & (RING_BYTES - 1);
-        read_stage_off = (read_stage_off + STAGE_BYTES) & (RING_BYTES - 1);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  };
-
-#pragma unroll
-  for (int c = 0; c < AHEAD; ++c) issue_chunk(c);
-  wait_loads_but<(AHEAD - 1) * LOADS>();
-  __syncthreads();
-#pragma unroll
-  for (int kk = 0; kk < 2; ++kk) {
-#pragma unroll
-    for (int j = 0; j < BN; ++j) pb[j][kk] = read_frag(A_PIECES, frag_b0 + j, kk);
-#pragma unroll
-    for (int i = 0; i < AM; ++i) pa[i][kk] = read_frag(0, frag_a0 + i, kk);
-  }
-  int kc = 0;
-  for (; kc + 1 < chunks; kc += 2) {
-    step(pa, pb, qa, qb);
-    step(qa, qb, pa, pb);
-  }
-  if (kc < chunks) step(pa, pb, qa, qb);
-  // No load may still be writing LDS when the workgroup's allocation is freed.
-  wait_loads_but<0>();
-
-  store_block<KIND, RHS_I4, AM, BN>(a, acc, first_row + wave_m * (32 * AM), first_col + wave_n * (32 * BN),
-                                    lane);
-}
 
 int log2_exact(int64_t v) {
   if (v <= 0 || (v & (v - 1))) return -1;
@@ -754,7 +16,8 @@ int log2_exact(int64_t v) {
 struct Plan {
   int kind;
   bool rhs_i4;
-  int gather;  // 16 or 4
+  bool narrow;  // 16-bit output, rounded once at the end
+  int gather;   // 16 or 4
   MfmaArgs args;
 };
 
@@ -762,12 +25,26 @@ struct Plan {
 // shape are looked at.
 bool make_plan(const Mmt4dArgs& a, bool probe_only, Plan* plan) {
   int kind, elem_bytes;
-  bool i4 = false;
+  bool i4 = false, narrow = false;
+  // With a 16-bit output the reference rounds the accumulator after every
+  // multiply-add unless told to skip that (mmt4d_tile_generic.c:229-286,
+  // 319-376): only the skipping variant (f32 accumulator, one rounding at the
+  // end) is something a matrix pipe can compute.
+  const bool skip_roundings = a.flags & IREE_UK_FLAG_MMT4D_SKIP_INTERMEDIATE_ROUNDINGS;
   switch (a.flags & IREE_UK_FLAG_MMT4D_TYPE_MASK) {
     case IREE_UK_FLAG_MMT4D_TYPE_S8S8S32: kind = kI8; elem_bytes = 1; break;
     case IREE_UK_FLAG_MMT4D_TYPE_S8S4S32: kind = kI8; elem_bytes = 1; i4 = true; break;
     case IREE_UK_FLAG_MMT4D_TYPE_F16F16F32: kind = kF16; elem_bytes = 2; break;
     case IREE_UK_FLAG_MMT4D_TYPE_BF16BF16F32: kind = kBF16; elem_bytes = 2; break;
+    case IREE_UK_FLAG_MMT4D_TYPE_F32F32F32: kind = kF32; elem_bytes = 4; break;
+    case IREE_UK_FLAG_MMT4D_TYPE_F16F16F16:
+      if (!skip_roundings) return false;
+      kind = kF16; elem_bytes = 2; narrow = true;
+      break;
+    case IREE_UK_FLAG_MMT4D_TYPE_BF16BF16BF16:
+      if (!skip_roundings) return false;
+      kind = kBF16; elem_bytes = 2; narrow = true;
+      break;
     default: return false;
   }
   const int lm0 = log2_exact(a.M0), ln0 = log2_exact(a.N0);
@@ -789,6 +66,7 @@ bool make_plan(const Mmt4dArgs& a, bool probe_only, Plan* plan) {
   }
   plan->kind = kind;
   plan->rhs_i4 = i4;
+  plan->narrow = narrow;
   plan->gather = gather;
   if (probe_only) return true;
 
@@ -823,122 +101,23 @@ bool make_plan(const Mmt4dArgs& a, bool probe_only, Plan* plan) {
   return true;
 }
 
-// Whether the direct-to-LDS kernel covers the problem: K ends on a chunk
-// boundary and every lane can load 16 contiguous bytes (4-byte row pieces 4
-// rows at a time, an int4 rhs in pieces of 32 nibbles).
-template <bool RHS_I4, int G>
-bool direct_covers(const MfmaArgs& m) {
-  if (((int64_t)m.K * m.lhs_rb) % 64 != 0) return false;
-  if (RHS_I4) return m.rhs_rb >= 16 && (uintptr_t)m.rhs % 16 == 0 && m.rhs_stride_bytes % 16 == 0;
-  if (G == 16) return true;
-  return m.log2_M0 >= 2 && m.log2_N0 >= 2 && (uintptr_t)m.lhs % 16 == 0 && (uintptr_t)m.rhs % 16 == 0 &&
-         m.lhs_stride_bytes % 16 == 0 && m.rhs_stride_bytes % 16 == 0;
-}
-
-void set_tile_grid(MfmaArgs* m, int block_rows, int block_cols, unsigned* grid) {
-  const int64_t rows = (int64_t)m->M << m->log2_M0, cols = (int64_t)m->N << m->log2_N0;
-  m->tile_rows = (int32_t)((rows + block_rows - 1) / block_rows);
-  m->tile_cols = (int32_t)((cols + block_cols - 1) / block_cols);
-  const int64_t tiles = (int64_t)m->tile_rows * m->tile_cols;
-  *grid = (unsigned)(((tiles + 7) / 8) * 8);
-}
-
-// Direct-to-LDS kernel on (64*AM) x (64*BN) block tiles with a ring of STAGES stages.
-template <int KIND, bool RHS_I4, int G, int AM, int BN, int STAGES>
-hipError_t launch_direct(MfmaArgs m, hipStream_t stream) {
-  unsigned grid;
-  set_tile_grid(&m, 64 * AM, 64 * BN, &grid);
-  constexpr int stage_pieces = 256 * AM + (RHS_I4 ? 128 : 256) * BN;
-  constexpr size_t lds_bytes = (size_t)STAGES * 16 * (stage_pieces <= 512 ? 512 : stage_pieces <= 1024 ? 1024 : 2048);
-  static_assert(lds_bytes <= 160 * 1024, "ring does not fit the LDS");
-  auto kernel = mmt4d_mfma_direct_kernel<KIND, RHS_I4, G, AM, BN, STAGES>;
-  // Above 64 KiB of dynamic LDS the limit has to be raised (per device, so it
-  // is simply done on every launch: it only sets a field).
-  if (lds_bytes > 65536) {
-    const hipError_t attr =
-        hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-    if (attr != hipSuccess) return attr;
-  }
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds_bytes, stream, m);
-  return hipGetLastError();
-}
-
-// Register-staged kernel (any K, any alignment the plan admits).
-template <int KIND, bool RHS_I4, int G, int AM, int BN, int MIN_BLOCKS>
-hipError_t launch_staged(MfmaArgs m, hipStream_t stream) {
-  unsigned grid;
-  set_tile_grid(&m, 64 * AM, 64 * BN, &grid);
-  // K ending inside a chunk needs the kernel variant with the zero-filling tail step.
-  const bool tail = ((int64_t)m.K * m.lhs_rb) % 64 != 0;
-  if (tail) {
-    hipLaunchKernelGGL((mmt4d_mfma_kernel<KIND, RHS_I4, G, AM, BN, MIN_BLOCKS, true>), dim3(grid),
-                       dim3(256), 0, stream, m);
-  } else {
-    hipLaunchKernelGGL((mmt4d_mfma_kernel<KIND, RHS_I4, G, AM, BN, MIN_BLOCKS, false>), dim3(grid),
-                       dim3(256), 0, stream, m);
-  }
-  return hipGetLastError();
-}
-
-// Picks the block tile. Every workgroup pulls its operands through L2 -> LDS at
-// a rate that does not depend on the tile, so the bytes moved per multiply
-// fall with the tile's size: the largest tile that still gives most compute
-// units a workgroup wins.
-template <int KIND, bool RHS_I4, int G>
-hipError_t launch_variant(const MfmaArgs& m, hipStream_t stream, const char** name) {
-  const int64_t rows = (int64_t)m.M << m.log2_M0, cols = (int64_t)m.N << m.log2_N0;
-  auto tiles = [&](int br, int bc) { return ((rows + br - 1) / br) * ((cols + bc - 1) / bc); };
-  const bool direct = direct_covers<RHS_I4, G>(m);
-  if (tiles(256, 256) >= 200) {
-    *name = "mmt4d_mfma_256x256";
-    if (direct) return launch_direct<KIND, RHS_I4, G, 4, 4, 4>(m, stream);
-    return launch_staged<KIND, RHS_I4, G, 4, 4, 1>(m, stream);
-  }
-  if (tiles(128, 128) >= 128) {
-    *name = "mmt4d_mfma_128x128";
-    if (direct) return launch_direct<KIND, RHS_I4, G, 2, 2, 4>(m, stream);
-    return launch_staged<KIND, RHS_I4, G, 2, 2, 2>(m, stream);
-  }
-  *name = "mmt4d_mfma_64x64";
-  if constexpr (!RHS_I4) {
-    if (direct) return launch_direct<KIND, RHS_I4, G, 1, 1, 8>(m, stream);
-  }
-  return launch_staged<KIND, RHS_I4, G, 1, 1, 2>(m, stream);
-}
-
 hipError_t launch_mfma(const Mmt4dArgs& a, hipStream_t stream, const char** name) {
   Plan plan;
   if (!make_plan(a, false, &plan)) return hipErrorInvalidValue;
   const MfmaArgs& m = plan.args;
-  if (plan.rhs_i4) return launch_variant<kI8, true, 16>(m, stream, name);
-  if (plan.kind == kI8)
-    return plan.gather == 16 ? launch_variant<kI8, false, 16>(m, stream, name)
-                             : launch_variant<kI8, false, 4>(m, stream, name);
-  if (plan.kind == kF16)
-    return plan.gather == 16 ? launch_variant<kF16, false, 16>(m, stream, name)
-                             : launch_variant<kF16, false, 4>(m, stream, name);
-  return plan.gather == 16 ? launch_variant<kBF16, false, 16>(m, stream, name)
-                           : launch_variant<kBF16, false, 4>(m, stream, name);
-}
-
-Mmt4dLauncher select_common(const Mmt4dArgs& a, bool probe_only, uint32_t type_a, uint32_t type_b) {
-  const uint32_t t = a.flags & IREE_UK_FLAG_MMT4D_TYPE_MASK;
-  if (t != type_a && t != type_b) return nullptr;
-  Plan plan;
-  return make_plan(a, probe_only, &plan) ? launch_mfma : nullptr;
+  switch (plan.kind) {
+    case kI8: return launch_mfma_i8(m, plan.gather, plan.rhs_i4, stream, name);
+    case kF16: return launch_mfma_f16(m, plan.gather, plan.narrow, stream, name);
+    case kBF16: return launch_mfma_bf16(m, plan.gather, plan.narrow, stream, name);
+    default: return launch_mfma_f32(m, plan.gather, stream, name);
+  }
 }
 
 }  // namespace
 
-Mmt4dLauncher select_mmt4d_i8_mfma(const Mmt4dArgs& a, bool probe_only) {
-  return select_common(a, probe_only, IREE_UK_FLAG_MMT4D_TYPE_S8S8S32, IREE_UK_FLAG_MMT4D_TYPE_S8S8S32);
-}
-Mmt4dLauncher select_mmt4d_f16_mfma(const Mmt4dArgs& a, bool probe_only) {
-  return select_common(a, probe_only, IREE_UK_FLAG_MMT4D_TYPE_F16F16F32,
-                       IREE_UK_FLAG_MMT4D_TYPE_BF16BF16F32);
-}
-Mmt4dLauncher select_mmt4d_s8s4_mfma(const Mmt4dArgs& a, bool probe_only) {
-  return select_common(a, probe_only, IREE_UK_FLAG_MMT4D_TYPE_S8S4S32, IREE_UK_FLAG_MMT4D_TYPE_S8S4S32);
+Mmt4dLauncher select_mmt4d_mfma(const Mmt4dArgs& a, bool probe_only) {
+  Plan plan;
+  return make_plan(a, probe_only, &plan) ? launch_mfma : nullptr;
 }
 
 }  // namespace uk

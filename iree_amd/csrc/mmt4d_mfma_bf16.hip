@@ -1,0 +1,16 @@
+// Kernel instantiations of the MFMA mmt4d for one operand type (see
+// mmt4d_mfma_kernels.h).
+#define UK_MFMA_KERNEL_BODIES
+#include "mmt4d_mfma_kernels.h"
+
+namespace uk {
+
+hipError_t launch_mfma_bf16(const MfmaArgs& m, int gather, bool narrow, hipStream_t stream, const char** name) {
+  if (narrow)
+    return gather == 16 ? launch_variant<kBF16, false, 16, true>(m, stream, name)
+                        : launch_variant<kBF16, false, 4, true>(m, stream, name);
+  return gather == 16 ? launch_variant<kBF16, false, 16, false>(m, stream, name)
+                      : launch_variant<kBF16, false, 4, false>(m, stream, name);
+}
+
+}  // namespace uk

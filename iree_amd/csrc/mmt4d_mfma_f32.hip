@@ -1,0 +1,13 @@
+// Kernel instantiations of the MFMA mmt4d for one operand type (see
+// mmt4d_mfma_kernels.h).
+#define UK_MFMA_KERNEL_BODIES
+#include "mmt4d_mfma_kernels.h"
+
+namespace uk {
+
+hipError_t launch_mfma_f32(const MfmaArgs& m, int gather, hipStream_t stream, const char** name) {
+  return gather == 16 ? launch_variant<kF32, false, 16, false>(m, stream, name)
+                      : launch_variant<kF32, false, 4, false>(m, stream, name);
+}
+
+}  // namespace uk

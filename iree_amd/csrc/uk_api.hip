@@ -161,9 +161,7 @@ bool launch_ok(hipError_t e, const char* what) {
 uk::Mmt4dLauncher select_mmt4d(const uk::Mmt4dArgs& a, bool probe_only) {
   uk::Mmt4dLauncher l = nullptr;
   if ((l = uk::select_mmt4d_gemv(a, probe_only))) return l;
-  if ((l = uk::select_mmt4d_i8_mfma(a, probe_only))) return l;
-  if ((l = uk::select_mmt4d_f16_mfma(a, probe_only))) return l;
-  if ((l = uk::select_mmt4d_s8s4_mfma(a, probe_only))) return l;
+  if ((l = uk::select_mmt4d_mfma(a, probe_only))) return l;
   return nullptr;
 }
 

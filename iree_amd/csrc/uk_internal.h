@@ -55,10 +55,8 @@ typedef hipError_t (*Mmt4dLauncher)(const Mmt4dArgs& a, hipStream_t stream, cons
 // Specialised mmt4d kernels. Each returns nullptr when it does not cover the
 // given problem (type, tile shape, alignment), else its launcher. `probe_only`
 // problems carry only type flags and M0/N0/K0 (used by iree_uk_mmt4d_info).
-Mmt4dLauncher select_mmt4d_i8_mfma(const Mmt4dArgs& a, bool probe_only);
-Mmt4dLauncher select_mmt4d_f16_mfma(const Mmt4dArgs& a, bool probe_only);
+Mmt4dLauncher select_mmt4d_mfma(const Mmt4dArgs& a, bool probe_only);
 Mmt4dLauncher select_mmt4d_gemv(const Mmt4dArgs& a, bool probe_only);
-Mmt4dLauncher select_mmt4d_s8s4_mfma(const Mmt4dArgs& a, bool probe_only);
 
 // One thread per output element; covers every type flag and tile shape.
 hipError_t launch_mmt4d_generic(const Mmt4dArgs& a, hipStream_t stream, const char** name);
