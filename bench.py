@@ -24,6 +24,7 @@ if ROOT not in sys.path:
 # Published MI355X peaks used for the roofline fractions.
 PEAK_INT8_TOPS = 5033.0     # dense int8 MFMA
 PEAK_F16_TFLOPS = 2516.0    # dense f16 / bf16 MFMA
+PEAK_F32_TFLOPS = 157.3     # dense f32 MFMA
 PEAK_HBM_GBS = 8000.0       # HBM3E
 
 # HBM traffic of ONE launch of the headline kernel, measured with the
@@ -137,6 +138,10 @@ def _also(torch, lib, abi, synth, steps, warmup):
     mm("mmt4d_f16f16f32_4096_16x16x16_acc", abi.MMT4D_TYPE_F16F16F32, 256, 256, 256, 16, 16, 16,
        f16_operand(3, 0, n, 1.0 / 64), f16_operand(3, 1, n, 1.0 / 64), torch.float32,
        PEAK_F16_TFLOPS, "TFLOP/s", acc=True)
+    # f32f32f32 4096^3 with the tile shape query_tile_sizes hands out for f32 (16x16x4).
+    mm("mmt4d_f32f32f32_4096_16x16x4", abi.MMT4D_TYPE_F32F32F32, 256, 256, 1024, 16, 16, 4,
+       torch.from_numpy(synth.normal_f32(6, 0, n, 1.0)).cuda(), torch.from_numpy(synth.normal_f32(6, 1, n, 1.0)).cuda(),
+       torch.float32, PEAK_F32_TFLOPS, "TFLOP/s")
     # s8s4s32 512 x 11008 x 4096, tiles 16x16x32.
     lhs = torch.from_numpy(synth.uniform_int8(5, 0, 512 * 4096)).cuda()
     rhs = torch.from_numpy(synth.uniform_int4_packed(5, 1, 11008 * 4096).view(np.int8)).cuda()

@@ -20,6 +20,10 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # The MFMA main loops are written as fully unrolled loops whose indices must
+    # be compile-time constants (register arrays); the f32 kernel's loop body is
+    # past the default size limit for `#pragma unroll`.
+    "-mllvm", "-pragma-unroll-threshold=1000000",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes",
 ]
 

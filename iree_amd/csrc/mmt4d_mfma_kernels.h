@@ -526,8 +526,12 @@ __device__ __forceinline__ void wait_loads_but() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
+// (The 256x256 tile needs all 512 registers of a lane for one wavefront; said
+// explicitly, because left to its occupancy heuristics the compiler may keep
+// the accumulators in scratch memory instead.)
 template <int KIND, bool RHS_I4, bool NARROW, int G, int AM, int BN, int STAGES>
-__global__ __launch_bounds__(256) void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, AM * BN >= 16 ? 1 : (AM * BN >= 4 ? 2 : 4))))
+void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   typedef typename AccType<KIND>::type acc_t;
   static_assert(!RHS_I4 || (G == 16 && BN >= 2), "int4 rhs: 16-byte pieces, at least one fragment per wavefront");
   constexpr int BLOCK_ROWS = 64 * AM, BLOCK_COLS = 64 * BN;
