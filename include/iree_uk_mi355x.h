@@ -233,8 +233,9 @@ void iree_uk_assert_fail(const char* file, int line, const char* function,
 int iree_uk_mi355x_version(void);
 
 /* Selects the HIP device for the calling thread's launches and checks that it
- * is a gfx950 part. Returns 0 on success, a HIP error code otherwise. Calling
- * it is optional: the first launch uses the current HIP device. */
+ * is a gfx950 part; a negative ordinal checks the thread's current device
+ * without selecting another. Returns 0 on success, a HIP error code otherwise.
+ * Calling it is optional: the first launch uses the current HIP device. */
 int iree_uk_mi355x_init(int device_ordinal);
 
 /* Per-thread launch mode.

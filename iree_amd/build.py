@@ -13,6 +13,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "build", "obj")
 LIB_PATH = os.path.join(HERE, "libiree_uk_mi355x.so")
+PLUGIN_PATH = os.path.join(HERE, "libiree_uk_mi355x_plugin.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 # Packed-FP32 instruction selection is switched off for every device
@@ -54,7 +55,21 @@ def build(verbose=False, jobs=8):
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stdout)
+    build_plugin()
     return LIB_PATH
+
+
+def build_plugin():
+    """The HAL executable plugin: plain C on top of the library's C ABI, found
+    next to it at run time ($ORIGIN)."""
+    cmd = ["gcc", "-O2", "-std=c11", "-Wall", "-Wextra", "-fPIC", "-shared", "-fvisibility=hidden",
+           "-I", os.path.join(os.path.dirname(HERE), "include"), "-I", os.path.join(CSRC, "plugin"),
+           os.path.join(CSRC, "plugin", "uk_plugin.c"), "-o", PLUGIN_PATH,
+           "-L", HERE, "-liree_uk_mi355x", "-Wl,-rpath,$ORIGIN"]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("plugin build failed:\n" + r.stdout)
+    return PLUGIN_PATH
 
 
 if __name__ == "__main__":

@@ -500,7 +500,7 @@ UK_API void iree_uk_query_tile_sizes_2d(const iree_uk_query_tile_sizes_2d_params
 UK_API int iree_uk_mi355x_version(void) { return 100; }
 
 UK_API int iree_uk_mi355x_init(int device_ordinal) {
-  hipError_t e = hipSetDevice(device_ordinal);
+  hipError_t e = device_ordinal < 0 ? hipGetDevice(&device_ordinal) : hipSetDevice(device_ordinal);
   if (e != hipSuccess) return (int)e;
   hipDeviceProp_t prop;
   e = hipGetDeviceProperties(&prop, device_ordinal);
