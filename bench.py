@@ -142,6 +142,19 @@ def _also(torch, lib, abi, synth, steps, warmup):
     mm("mmt4d_f32f32f32_4096_16x16x4", abi.MMT4D_TYPE_F32F32F32, 256, 256, 1024, 16, 16, 4,
        torch.from_numpy(synth.normal_f32(6, 0, n, 1.0)).cuda(), torch.from_numpy(synth.normal_f32(6, 1, n, 1.0)).cuda(),
        torch.float32, PEAK_F32_TFLOPS, "TFLOP/s")
+    # The in-dispatch int8 microkernel (16x16x64 MFMA, data-tiled operands of the
+    # GPU backend's layout) over a 16 x 16 grid of 256x256 tiles, K = 4096; it
+    # accumulates into C, which is therefore read and written.
+    ta = torch.from_numpy(synth.uniform_int8(7, 0, n)).cuda()
+    tb = torch.from_numpy(synth.uniform_int8(7, 1, n)).cuda()
+    tc = torch.zeros(n, dtype=torch.int32, device="cuda")
+    ms, _ = _time_launches(torch, lambda: lib.iree_uk_mi355x_multi_mma_i32_16x16x64_i8(
+        ta.data_ptr(), tb.data_ptr(), tc.data_ptr(), 16, 16, 64, 8, 2, 8, 2, 1), steps, warmup)
+    res["multi_mma_i32_16x16x64_i8_4096_device_ukernel"] = {
+        "kernel": lib.iree_uk_mi355x_last_kernel().decode(), "ms": round(ms, 5),
+        "value": round(2.0 * 4096 ** 3 / ms / 1e9, 1), "unit": "TOP/s",
+        "frac_of_peak": round(2.0 * 4096 ** 3 / ms / 1e9 / PEAK_INT8_TOPS, 4)}
+    del ta, tb, tc
     # s8s4s32 512 x 11008 x 4096, tiles 16x16x32.
     lhs = torch.from_numpy(synth.uniform_int8(5, 0, 512 * 4096)).cuda()
     rhs = torch.from_numpy(synth.uniform_int4_packed(5, 1, 11008 * 4096).view(np.int8)).cuda()

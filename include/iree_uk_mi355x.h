@@ -229,6 +229,26 @@ void iree_uk_assert_fail(const char* file, int line, const char* function,
 /* Entry points without a counterpart in the reference.                       */
 /*===--------------------------------------------------------------------===*/
 
+/* The in-dispatch int8 microkernel of the ROCm backend's calling convention
+ * for gfx950 (iree_amd/csrc/device/iree_uk_amdgpu_multi_mma_mfma_i32_16x16x64_i8.h;
+ * the reference has the gfx942 one, compiler/plugins/target/ROCM/builtins/
+ * ukernel/iree_uk_amdgpu_multi_mma_mfma_i32_16x16x32_i8.c:82-181), run over a
+ * grid of outer_m x outer_n data-tiled tiles, one workgroup each:
+ *   a: [outer_m][k_size][subgroups_m][intrinsics_m][64][intrinsics_k] vectors of 16 int8,
+ *   b: [outer_n][k_size][subgroups_n][intrinsics_n][64][intrinsics_k],
+ *   c: [outer_m][outer_n][subgroups_m][subgroups_n][intrinsics_m][intrinsics_n][64] vectors of 4 int32,
+ * c += a * b^T in the MFMA's operand layout (lane l of an A/B vector block: row
+ * l % 16, K bytes 16*(l / 16)..+15 of 64; lane l of a C block: rows
+ * 4*(l / 16)+{0..3}, column l % 16). Device pointers only. The parameter
+ * combinations are compile-time instantiations; returns 0, or a HIP error
+ * code (hipErrorInvalidValue for a combination that is not instantiated). It
+ * exists to test and measure the device microkernel; there is no host entry
+ * point like it in the reference. */
+int iree_uk_mi355x_multi_mma_i32_16x16x64_i8(const void* a, const void* b, void* c, long long outer_m,
+                                             long long outer_n, int32_t k_size, int32_t intrinsics_m,
+                                             int32_t subgroups_m, int32_t intrinsics_n, int32_t subgroups_n,
+                                             int32_t intrinsics_k);
+
 /* Library version, MAJOR*10000 + MINOR*100 + PATCH. */
 int iree_uk_mi355x_version(void);
 

@@ -497,6 +497,24 @@ UK_API void iree_uk_query_tile_sizes_2d(const iree_uk_query_tile_sizes_2d_params
 // Entry points without a reference counterpart
 //===----------------------------------------------------------------------===//
 
+UK_API int iree_uk_mi355x_multi_mma_i32_16x16x64_i8(const void* a, const void* b, void* c, long long outer_m,
+                                                    long long outer_n, int32_t k_size, int32_t intrinsics_m,
+                                                    int32_t subgroups_m, int32_t intrinsics_n, int32_t subgroups_n,
+                                                    int32_t intrinsics_k) {
+  tl_last_kernel = "";
+  // Device pointers only: the data-tiled operands of a GPU dispatch never live on the host.
+  if (!device_accessible(a) || !device_accessible(b) || !device_accessible(c)) return (int)hipErrorInvalidValue;
+  const hipError_t e = uk::launch_multi_mma_i8(a, b, c, outer_m, outer_n, k_size, intrinsics_m, subgroups_m,
+                                               intrinsics_n, subgroups_n, intrinsics_k, tl_stream);
+  if (e != hipSuccess) return (int)e;
+  tl_last_kernel = "multi_mma_i32_16x16x64_i8";
+  if (!tl_async) {
+    const hipError_t s = hipStreamSynchronize(tl_stream);
+    if (s != hipSuccess) return (int)s;
+  }
+  return 0;
+}
+
 UK_API int iree_uk_mi355x_version(void) { return 100; }
 
 UK_API int iree_uk_mi355x_init(int device_ordinal) {

@@ -58,6 +58,11 @@ typedef hipError_t (*Mmt4dLauncher)(const Mmt4dArgs& a, hipStream_t stream, cons
 Mmt4dLauncher select_mmt4d_mfma(const Mmt4dArgs& a, bool probe_only);
 Mmt4dLauncher select_mmt4d_gemv(const Mmt4dArgs& a, bool probe_only);
 
+// The in-dispatch int8 microkernel over a grid of data-tiled tiles (multi_mma.hip).
+hipError_t launch_multi_mma_i8(const void* a, const void* b, void* c, int64_t outer_m, int64_t outer_n, int32_t k_size,
+                               int intrinsics_m, int subgroups_m, int intrinsics_n, int subgroups_n, int intrinsics_k,
+                               hipStream_t stream);
+
 // One thread per output element; covers every type flag and tile shape.
 hipError_t launch_mmt4d_generic(const Mmt4dArgs& a, hipStream_t stream, const char** name);
 

@@ -49,6 +49,8 @@ def load():
                                               C.POINTER(abi.QueryTileSizes2dOutParams)]
     l.iree_uk_query_tile_sizes_2d.restype = None
     l.iree_uk_mi355x_version.restype = C.c_int
+    l.iree_uk_mi355x_multi_mma_i32_16x16x64_i8.argtypes = [vp, vp, vp, C.c_longlong, C.c_longlong] + [C.c_int32] * 6
+    l.iree_uk_mi355x_multi_mma_i32_16x16x64_i8.restype = C.c_int
     l.iree_uk_mi355x_init.argtypes = [C.c_int]
     l.iree_uk_mi355x_init.restype = C.c_int
     l.iree_uk_mi355x_set_stream.argtypes = [vp, C.c_int]
