@@ -537,13 +537,9 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   constexpr int BLOCK_ROWS = 64 * AM, BLOCK_COLS = 64 * BN;
   // 16-byte pieces per chunk: 64 bytes of K per row, 32 bytes for an int4 rhs.
   constexpr int A_PIECES = BLOCK_ROWS * 4, B_PIECES = BLOCK_COLS * (RHS_I4 ? 2 : 4);
-  // Stage size rounded up to a power of two so that ring offsets wrap with a mask.
-  constexpr int STAGE_PIECES = A_PIECES + B_PIECES <= 512    ? 512
-                               : A_PIECES + B_PIECES <= 1024 ? 1024
-                                                             : 2048;
-  static_assert(A_PIECES + B_PIECES <= STAGE_PIECES, "stage too small");
+  constexpr int STAGE_PIECES = A_PIECES + B_PIECES;
   constexpr int AHEAD = STAGES - 1;  // chunks in flight ahead of the one being multiplied
-  static_assert(STAGES >= 4 && (STAGES & (STAGES - 1)) == 0, "ring depth");
+  static_assert(STAGES >= 4, "ring depth");
   // Load instructions per wavefront and chunk (64 lanes x 16 bytes each), each
   // with its own per-lane offset.
   constexpr int A_LOADS = A_PIECES / 256, B_LOADS = B_PIECES / 256;
@@ -651,7 +647,7 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   };
   auto issue_chunk = [&](int kc) {
     const int idx = min(kc, last_chunk);
-    const uint32_t stage_off = (uint32_t)(kc & (STAGES - 1)) * (STAGE_PIECES * 16);
+    const uint32_t stage_off = (uint32_t)(kc % STAGES) * (STAGE_PIECES * 16);
     const uint8_t* la = lhs_base + idx * lhs_chunk_bytes + lhs_wave_bytes;
     const uint8_t* lb = rhs_base + idx * rhs_chunk_bytes + rhs_wave_bytes;
 #pragma unroll
@@ -680,7 +676,6 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   // chunk number (64-bit multiplies on the scalar unit, in front of the step's
   // first MFMA).
   constexpr uint32_t STAGE_BYTES = STAGE_PIECES * 16, RING_BYTES = STAGES * STAGE_BYTES;
-  static_assert((RING_BYTES & (RING_BYTES - 1)) == 0, "ring offsets wrap with a mask");
   const uint8_t* load_a = lhs_base + min(AHEAD, last_chunk) * lhs_chunk_bytes + lhs_wave_bytes;
   const uint8_t* load_b = rhs_base + min(AHEAD, last_chunk) * rhs_chunk_bytes + rhs_wave_bytes;
   int load_chunk = AHEAD;
@@ -778,8 +773,8 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
         load_a += more ? lhs_chunk_bytes : 0;
         load_b += more ? rhs_chunk_bytes : 0;
         ++load_chunk;
-        load_stage_off = (load_stage_off + STAGE_BYTES) & (RING_BYTES - 1);
-        read_stage_off = (read_stage_off + STAGE_BYTES) & (RING_BYTES - 1);
+        load_stage_off = load_stage_off + STAGE_BYTES == RING_BYTES ? 0 : load_stage_off + STAGE_BYTES;
+        read_stage_off = read_stage_off + STAGE_BYTES == RING_BYTES ? 0 : read_stage_off + STAGE_BYTES;
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -835,7 +830,7 @@ hipError_t launch_direct(MfmaArgs m, hipStream_t stream) {
   unsigned grid;
   set_tile_grid(&m, 64 * AM, 64 * BN, &grid);
   constexpr int stage_pieces = 256 * AM + (RHS_I4 ? 128 : 256) * BN;
-  constexpr size_t lds_bytes = (size_t)STAGES * 16 * (stage_pieces <= 512 ? 512 : stage_pieces <= 1024 ? 1024 : 2048);
+  constexpr size_t lds_bytes = (size_t)STAGES * 16 * stage_pieces;
   static_assert(lds_bytes <= 160 * 1024, "ring does not fit the LDS");
   auto kernel = mmt4d_mfma_direct_kernel<KIND, RHS_I4, NARROW, G, AM, BN, STAGES>;
   // Above 64 KiB of dynamic LDS the limit has to be raised (per device, so it
