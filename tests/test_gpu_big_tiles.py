@@ -1,0 +1,130 @@
+"""The large block tiles of the MFMA kernels (256x256 and 128x128 per
+workgroup) on shapes that do not divide into them: ragged last block rows and
+columns, K that ends inside a 64-byte chunk, strided operands with offsets,
+accumulation. The reference's own test grid only reaches the smallest block
+tile; the benchmark configurations only exact multiples.
+
+Integer results are compared bit for bit with a float64 matrix product of the
+same operands (every value is far below 2^53, so that product is exact); float
+results within |got - ref| <= 1e-3 * max(|ref|, rms(ref)) of it.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from iree_amd import abi
+from test_gpu_configs import REL_TOL, gpu_lib, mm_params  # noqa: F401
+
+pytestmark = pytest.mark.gpu
+
+
+def logical(t, outer, K, T0, K0):
+    """[outer][K][T0][K0] tiled operand -> [outer*T0, K*K0] float64."""
+    return t.view(outer, K, T0, K0).permute(0, 2, 1, 3).reshape(outer * T0, K * K0).double()
+
+
+def run_case(gpu_lib, flags, M, N, K, M0, N0, K0, expect_kernel, lhs_pad=0, rhs_pad=0, out_pad=0, offsets=(0, 0, 0),
+             accumulate=False, seed=0):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    kind = flags & 0xFF
+    lhs_stride, rhs_stride, out_stride = K * M0 * K0 + lhs_pad, K * N0 * K0 + rhs_pad, N * M0 * N0 + out_pad
+    lo, ro, oo = offsets
+
+    def operand(n_tiles, stride, off, T0):
+        if kind in (abi.MMT4D_TYPE_S8S8S32, abi.MMT4D_TYPE_S8S4S32):
+            return torch.randint(-128, 128, (off + n_tiles * stride,), dtype=torch.int8, device="cuda", generator=g)
+        dt = {abi.MMT4D_TYPE_F16F16F32: torch.float16, abi.MMT4D_TYPE_BF16BF16F32: torch.bfloat16,
+              abi.MMT4D_TYPE_F32F32F32: torch.float32}[kind]
+        return (torch.randn(off + n_tiles * stride, device="cuda", generator=g) / 8).to(dt)
+
+    lhs = operand(M, lhs_stride, lo, M0)
+    if kind == abi.MMT4D_TYPE_S8S4S32:
+        # packed nibbles: strides and offsets are in 4-bit elements
+        rhs_bytes = torch.randint(-128, 128, ((ro + N * rhs_stride) // 2,), dtype=torch.int8, device="cuda", generator=g)
+        rhs = rhs_bytes
+    else:
+        rhs = operand(N, rhs_stride, ro, N0)
+    is_int = kind in (abi.MMT4D_TYPE_S8S8S32, abi.MMT4D_TYPE_S8S4S32)
+    out_dtype = torch.int32 if is_int else torch.float32
+    if is_int:
+        out = torch.randint(-1000, 1000, (oo + M * out_stride,), dtype=torch.int32, device="cuda", generator=g)
+    else:
+        out = torch.randn(oo + M * out_stride, device="cuda", generator=g)
+    before = out.clone()
+    p = mm_params(lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), M, N, K, M0, N0, K0,
+                  flags | (abi.MMT4D_ACCUMULATE if accumulate else 0), lhs_off=lo, rhs_off=ro, out_off=oo,
+                  lhs_stride=lhs_stride, rhs_stride=rhs_stride, out_stride=out_stride)
+    gpu_lib.iree_uk_mmt4d_p(C.byref(p))
+    assert gpu_lib.iree_uk_mi355x_last_kernel() == expect_kernel.encode()
+
+    def rows_of(buf, off, n_tiles, stride, width):
+        return buf[off:off + n_tiles * stride].view(n_tiles, stride)[:, :width]
+
+    a = logical(rows_of(lhs, lo, M, lhs_stride, K * M0 * K0).contiguous(), M, K, M0, K0)
+    if kind == abi.MMT4D_TYPE_S8S4S32:
+        nib = rhs_bytes[ro // 2:(ro + N * rhs_stride) // 2].view(N, rhs_stride // 2)[:, :K * N0 * K0 // 2].contiguous()
+        u = nib.view(torch.uint8).to(torch.int16)
+        low = ((u & 0xF) ^ 8) - 8
+        high = ((u >> 4) ^ 8) - 8
+        vals = torch.stack([low, high], dim=-1).reshape(N, K * N0 * K0)
+        b = logical(vals, N, K, N0, K0)
+    else:
+        b = logical(rows_of(rhs, ro, N, rhs_stride, K * N0 * K0).contiguous(), N, K, N0, K0)
+    ref = a @ b.t()
+    if accumulate:
+        c0 = rows_of(before, oo, M, out_stride, N * M0 * N0).reshape(M, N, M0, N0).permute(0, 2, 1, 3).reshape(M * M0, N * N0)
+        ref = ref + c0.double()
+    got = rows_of(out, oo, M, out_stride, N * M0 * N0).reshape(M, N, M0, N0).permute(0, 2, 1, 3).reshape(M * M0, N * N0)
+    if is_int:
+        assert torch.equal(got.long(), ref.long())
+    else:
+        rms = ref.pow(2).mean().sqrt()
+        assert bool(((got.double() - ref).abs() <= REL_TOL * torch.maximum(ref.abs(), rms)).all())
+    # Nothing outside the output tiles was written: the gaps between tile rows and the prefix.
+    if out_pad:
+        gaps = out[oo:oo + M * out_stride].view(M, out_stride)[:, N * M0 * N0:]
+        assert torch.equal(gaps, before[oo:oo + M * out_stride].view(M, out_stride)[:, N * M0 * N0:])
+    assert torch.equal(out[:oo], before[:oo])
+
+
+# (M, N) in tiles chosen so that 256x256 blocks give >= 200 workgroups with a ragged last row and column.
+@pytest.mark.parametrize("K,accumulate", [(48, False), (40, True), (16, True)])
+def test_s8s8s32_8x8x4_ragged_256(gpu_lib, K, accumulate):
+    run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, 451, 463, K, 8, 8, 4, "mmt4d_mfma_256x256", accumulate=accumulate, seed=K)
+
+
+def test_s8s8s32_8x8x4_ragged_256_strided_with_offsets(gpu_lib):
+    # pads keep every tile row 16-byte aligned (the direct kernel), offsets are multiples of 16 elements
+    run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, 451, 463, 48, 8, 8, 4, "mmt4d_mfma_256x256", lhs_pad=64, rhs_pad=32,
+             out_pad=12, offsets=(32, 48, 8), accumulate=True, seed=3)
+    # 4-byte aligned only: the register-staged kernel
+    run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, 451, 463, 48, 8, 8, 4, "mmt4d_mfma_256x256", lhs_pad=4, rhs_pad=12,
+             out_pad=4, offsets=(4, 20, 4), seed=4)
+
+
+@pytest.mark.parametrize("M0,N0,K0,K", [(16, 16, 64, 3), (16, 8, 16, 9), (4, 16, 32, 5)])
+def test_s8s8s32_wide_pieces_ragged_256(gpu_lib, M0, N0, K0, K):
+    M, N = 3608 // M0 + 1, 3704 // N0 + 1
+    run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, M, N, K, M0, N0, K0, "mmt4d_mfma_256x256", accumulate=True, seed=K0)
+
+
+@pytest.mark.parametrize("M,N", [(100, 119), (131, 67)])
+def test_s8s8s32_ragged_128(gpu_lib, M, N):
+    run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, M, N, 32, 16, 16, 16, "mmt4d_mfma_128x128", out_pad=20, accumulate=True, seed=M)
+    run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, 2 * M, 2 * N, 19, 8, 8, 4, "mmt4d_mfma_128x128", seed=N)
+
+
+@pytest.mark.parametrize("flags,M0,N0,K0,K", [(abi.MMT4D_TYPE_F16F16F32, 16, 16, 16, 10), (abi.MMT4D_TYPE_BF16BF16F32, 16, 16, 8, 13),
+                                              (abi.MMT4D_TYPE_F16F16F32, 8, 8, 2, 48), (abi.MMT4D_TYPE_F32F32F32, 16, 16, 4, 11),
+                                              (abi.MMT4D_TYPE_F32F32F32, 8, 8, 1, 33)])
+def test_float_types_ragged_256(gpu_lib, flags, M0, N0, K0, K):
+    M, N = 3608 // M0 + 1, 3704 // N0 + 1
+    run_case(gpu_lib, flags, M, N, K, M0, N0, K0, "mmt4d_mfma_256x256", accumulate=True, out_pad=16, seed=K)
+
+
+@pytest.mark.parametrize("M,N,expect", [(226, 232, "mmt4d_mfma_256x256"), (100, 119, "mmt4d_mfma_128x128"), (9, 11, "mmt4d_mfma_64x64")])
+def test_s8s4s32_ragged(gpu_lib, M, N, expect):
+    run_case(gpu_lib, abi.MMT4D_TYPE_S8S4S32, M, N, 6, 16, 16, 32, expect, accumulate=True, rhs_pad=64, offsets=(16, 64, 4), seed=M)
+    run_case(gpu_lib, abi.MMT4D_TYPE_S8S4S32, M, N, 5, 16, 16, 16, expect, seed=N)   # 8-byte rhs pieces: staged kernel
