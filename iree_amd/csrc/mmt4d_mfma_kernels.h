@@ -571,9 +571,15 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
 
   // Load t of wavefront w fills the 16-byte LDS slots 64*m .. 64*m + 63 of its
   // operand, m = 4*t + w, lane l the slot 64*m + l.
-  //   G == 16: slot p holds fragment p >> 7, 16-byte column (p >> 5) & 3 (K-step
-  //     c >> 1, lane half c & 1 of the MFMA operand), row p & 31: a fragment is
-  //     read back with one 128-bit read at slot 128*f + 64*kk + lane.
+  //   G == 16: slot p holds fragment p >> 7, rows 16*((p >> 6) & 1) + (p & 15),
+  //     16-byte column c = (p >> 4) & 3 (K-step c >> 1, lane half c & 1 of the
+  //     MFMA operand): one load covers 16 rows x 64 bytes, which for 64-byte row
+  //     pieces is 1 KiB of contiguous memory (with "32 rows x 32 bytes" every
+  //     cache line was touched by two loads: 7 % slower). Lane 32*h + r reads
+  //     slot 128*f + 64*(r >> 4) + 16*(2*kk + h) + (r & 15), one 128-bit read;
+  //     every group of 16 lanes reads 256 contiguous bytes: no bank conflicts.
+  //     (With an int4 rhs the lhs keeps the older arrangement: slot p holds row
+  //     p & 31, column slot (p >> 5) & 3, read at slot 128*f + 64*kk + lane.)
   //   G == 4: slot 64*m + l holds rows 4*g .. 4*g + 3 (g = l & 7) of fragment
   //     m >> 1 at k step 8*(m & 1) + 4*h + d of the chunk (h = (l >> 3) & 1,
   //     d = l >> 4). Dword 64*(8*f + 4*kk + d) + 32*h + r of the operand is then
@@ -597,16 +603,17 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
 #pragma unroll
     for (int t = 0; t < A_LOADS; ++t) {
       const int p = tid + 256 * t;
-      const int c = RHS_I4 ? ((p >> 6) & 1) + 2 * ((p >> 5) & 1) : (p >> 5) & 3;
-      a_off[t] = (uint32_t)(row_offset(first_row + (p >> 7) * 32 + (p & 31), total_rows - 1, first_row,
+      const int c = RHS_I4 ? ((p >> 6) & 1) + 2 * ((p >> 5) & 1) : (p >> 4) & 3;
+      const int row = RHS_I4 ? (p >> 7) * 32 + (p & 31) : (p >> 7) * 32 + 16 * ((p >> 6) & 1) + (p & 15);
+      a_off[t] = (uint32_t)(row_offset(first_row + row, total_rows - 1, first_row,
                                        a.log2_M0, a.lhs_stride_bytes, a.lhs_rb) +
                             ((16 * c) >> a.log2_lhs_rb) * lhs_kstep + ((16 * c) & (a.lhs_rb - 1)));
     }
 #pragma unroll
     for (int t = 0; t < B_LOADS; ++t) {
       const int p = tid + 256 * t;
-      const int c = RHS_I4 ? (p >> 5) & 1 : (p >> 5) & 3;
-      const int row = RHS_I4 ? (p >> 6) * 32 + (p & 31) : (p >> 7) * 32 + (p & 31);
+      const int c = RHS_I4 ? (p >> 5) & 1 : (p >> 4) & 3;
+      const int row = RHS_I4 ? (p >> 6) * 32 + (p & 31) : (p >> 7) * 32 + 16 * ((p >> 6) & 1) + (p & 15);
       b_off[t] = (uint32_t)(row_offset(first_col + row, total_cols - 1, first_col, a.log2_N0,
                                        a.rhs_stride_bytes, a.rhs_rb) +
                             ((16 * c) >> a.log2_rhs_rb) * rhs_kstep + ((16 * c) & (a.rhs_rb - 1)));
@@ -662,6 +669,7 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
       return widen_i4_times16(kk ? make_uint2(raw.z, raw.w) : make_uint2(raw.x, raw.y));
     }
     if constexpr (G == 16) {
+      if (!RHS_I4) return ring[operand + 128 * f + 32 * kk + 64 * ((lane & 31) >> 4) + 16 * (lane >> 5) + (lane & 15)];
       return ring[operand + 128 * f + 64 * kk + lane];
     } else {
       const uint32_t* words = (const uint32_t*)(ring + operand) + 64 * (8 * f + 4 * kk) + lane;
@@ -683,7 +691,13 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   uint32_t read_stage_off = STAGE_BYTES;
   const uint32_t frag_a_off = (uint32_t)((wave_m * AM) * 128) * 16;
   const uint32_t frag_b_off = (uint32_t)(A_PIECES + (wave_n * BN) * (RHS_I4 ? 64 : 128)) * 16;
-  const uint8_t* ring_bytes = (const uint8_t*)ring + (G == 16 ? 16 : 4) * lane;
+  // Lane 32*h + r's byte offset into a fragment, and the slots from one K-step
+  // of a fragment to the next (see the layouts above).
+  constexpr bool ROWS16 = G == 16 && !RHS_I4;
+  const uint8_t* ring_bytes =
+      (const uint8_t*)ring + (ROWS16 ? 16 * (64 * ((lane & 31) >> 4) + 16 * (lane >> 5) + (lane & 15))
+                                     : (G == 16 ? 16 : 4) * lane);
+  constexpr int KK16 = ROWS16 ? 32 : 64;
 
   // One pipeline step for the chunk whose fragments are in `cur`:
   //   a few MFMAs first (they only need registers, and keep the matrix pipe
@@ -739,7 +753,7 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
               raw_b[u] = *(const uint4*)(read_b + (64 * u) * 16);
             } else {
               const int kk = (u - B_UNITS) / AM, i = (u - B_UNITS) % AM;
-              nxt_a[i][kk] = *(const uint4*)(read_a + (128 * i + 64 * kk) * 16);
+              nxt_a[i][kk] = *(const uint4*)(read_a + (128 * i + KK16 * kk) * 16);
             }
           } else {
             const int f = u / PARTS, part = u % PARTS;
@@ -748,7 +762,7 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
             const uint8_t* src = e < BN ? read_b : read_a;
             const int frag = e < BN ? e : e - BN;
             if constexpr (G == 16) {
-              dst = *(const uint4*)(src + (128 * frag + 64 * kk) * 16);
+              dst = *(const uint4*)(src + (128 * frag + KK16 * kk) * 16);
             } else {
               const uint32_t* words = (const uint32_t*)src + 64 * (8 * frag + 4 * kk + 2 * part);
               if (part == 0) { dst.x = words[0]; dst.y = words[64]; }
