@@ -322,6 +322,51 @@ def _cpu_baseline(abi, synth, threads):
     return base, extra
 
 
+def _cpu_pack_unpack(abi, synth, threads):
+    """The reference's pack and unpack on this host (f32 [8191, 8190] <-> [512, 8190, 16, 1],
+    rows of tiles split over `threads`), GB/s counted like the GPU figures (read + written)."""
+    import numpy as np
+    import oracle
+    ref = oracle.ref_lib()
+    if ref is None:
+        return None
+    R, Cc = 8191, 8190
+    src = synth.normal_f32(2, 0, R * Cc)
+    packed = np.empty(512 * Cc * 16, dtype=np.float32)
+    back = np.empty(R * Cc, dtype=np.float32)
+    cpu = oracle.host_cpu_data()
+    p = abi.PackParams()
+    p.in_buffer, p.out_buffer = src.ctypes.data, packed.ctypes.data
+    p.in_stride0, p.in_stride1, p.out_stride0, p.out_stride1 = Cc, 1, Cc * 16, 16
+    p.in_size0, p.in_size1 = R, Cc
+    p.out_size0, p.out_size1, p.out_size2, p.out_size3 = 512, Cc, 16, 1
+    p.padding_value, p.flags = 0, abi.PACK_TYPE_F32F32
+    p.cpu_data = C.cast(cpu, C.POINTER(C.c_uint64))
+    u = abi.UnpackParams()
+    u.in_buffer, u.out_buffer = packed.ctypes.data, back.ctypes.data
+    u.in_stride0, u.in_stride1, u.out_stride0, u.out_stride1 = Cc * 16, 16, Cc, 1
+    u.in_size0, u.in_size1, u.in_size2, u.in_size3 = 512, Cc, 16, 1
+    u.out_size0, u.out_size1, u.flags = R, Cc, abi.UNPACK_TYPE_F32F32
+    u.cpu_data = C.cast(cpu, C.POINTER(C.c_uint64))
+
+    def best_of(fn, n=3):
+        best = None
+        for _ in range(n):
+            t0 = time.perf_counter()
+            fn()
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        return best
+    t_pack = best_of(lambda: ref.ref_pack_mt(C.byref(p), threads))
+    t_unpack = best_of(lambda: ref.ref_unpack_mt(C.byref(u), threads))
+    return {"pack_f32_8191x8190_to_512x8190x16x1": {"value": round((R * Cc + 512 * Cc * 16) * 4 / t_pack / 1e9, 2),
+                                                   "unit": "GB/s", "cores": threads, "kind": "reference"},
+            "unpack_f32_512x8190x16x1_to_8191x8190": {"value": round(2 * R * Cc * 4 / t_unpack / 1e9, 2),
+                                                      "unit": "GB/s", "cores": threads, "kind": "reference"},
+            "round_trip_bit_exact": bool(np.array_equal(src, back)),
+            "sample": "the whole workload, best of 3"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -395,6 +440,10 @@ def main():
     }
     if cpu_arch is not None:
         line["cpu_baseline_arch_tiles"] = cpu_arch
+    if not args.no_cpu and not args.no_also:
+        cpu_pack = _cpu_pack_unpack(abi, synth, threads)
+        if cpu_pack is not None:
+            line["cpu_baseline_pack_unpack"] = cpu_pack
     if also is not None:
         line["also"] = also
     print(json.dumps(line))
