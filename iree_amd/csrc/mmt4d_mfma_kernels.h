@@ -875,30 +875,70 @@ hipError_t launch_staged(MfmaArgs m, hipStream_t stream) {
   return hipGetLastError();
 }
 
-// Picks the block tile. Every workgroup pulls its operands through L2 -> LDS at
-// a rate that does not depend on the tile, so the bytes moved per multiply
-// fall with the tile's size: the largest tile that still gives most compute
-// units a workgroup wins.
+// Picks the block tile. Larger tiles move fewer operand bytes per multiply
+// through L2 -> LDS and run the matrix pipe longer between barriers, smaller
+// ones spread a problem over more compute units. The estimate is
+//   (workgroups per compute unit, rounded up) x (tile area) / (tile efficiency),
+// with the efficiencies measured at saturation on bf16 16x16x8 operands
+// (TFLOP/s at 2048 x 14336 x 4096: 256x256 1003, 256x128 905, 128x128 851,
+// 128x64 607, 64x64 529). It reproduces the measured best tile on every shape
+// tried (128 .. 4096 rows against 14336 columns, 1024^2 .. 4096^2 squares).
+struct TileChoice {
+  int am, bn;
+  float efficiency;
+  bool direct_only;  // no register-staged instantiation of this shape
+};
+
+template <bool RHS_I4>
+int choose_tile(const MfmaArgs& m, bool direct, const TileChoice** chosen) {
+  static const TileChoice kTiles[] = {
+      {4, 4, 1003.f, false}, {4, 2, 905.f, true}, {2, 2, 851.f, false}, {2, 1, 607.f, true}, {1, 1, 529.f, false}};
+  const int64_t rows = (int64_t)m.M << m.log2_M0, cols = (int64_t)m.N << m.log2_N0;
+  int best = -1;
+  double best_cost = 0;
+  for (int i = 0; i < (int)(sizeof kTiles / sizeof kTiles[0]); ++i) {
+    const TileChoice& t = kTiles[i];
+    if (t.direct_only && !direct) continue;
+    if (RHS_I4 && t.bn < 2 && t.direct_only) continue;  // the int4 direct path needs a rhs fragment per wavefront
+    const int64_t br = 64 * t.am, bc = 64 * t.bn;
+    const int64_t workgroups = ((rows + br - 1) / br) * ((cols + bc - 1) / bc);
+    const double cost = (double)((workgroups + 255) / 256) * (double)(br * bc) / t.efficiency;
+    if (best < 0 || cost < best_cost) {
+      best = i;
+      best_cost = cost;
+    }
+  }
+  *chosen = &kTiles[best];
+  return best;
+}
+
 template <int KIND, bool RHS_I4, int G, bool NARROW>
 hipError_t launch_variant(const MfmaArgs& m, hipStream_t stream, const char** name) {
-  const int64_t rows = (int64_t)m.M << m.log2_M0, cols = (int64_t)m.N << m.log2_N0;
-  auto tiles = [&](int br, int bc) { return ((rows + br - 1) / br) * ((cols + bc - 1) / bc); };
   const bool direct = direct_covers<RHS_I4, G>(m);
-  if (tiles(256, 256) >= 200) {
-    *name = "mmt4d_mfma_256x256";
-    if (direct) return launch_direct<KIND, RHS_I4, NARROW, G, 4, 4, 4>(m, stream);
-    return launch_staged<KIND, RHS_I4, NARROW, G, 4, 4, 1>(m, stream);
+  const TileChoice* tile;
+  switch (choose_tile<RHS_I4>(m, direct, &tile)) {
+    case 0:
+      *name = "mmt4d_mfma_256x256";
+      if (direct) return launch_direct<KIND, RHS_I4, NARROW, G, 4, 4, 4>(m, stream);
+      return launch_staged<KIND, RHS_I4, NARROW, G, 4, 4, 1>(m, stream);
+    case 1:
+      *name = "mmt4d_mfma_256x128";
+      return launch_direct<KIND, RHS_I4, NARROW, G, 4, 2, 4>(m, stream);
+    case 2:
+      *name = "mmt4d_mfma_128x128";
+      if (direct) return launch_direct<KIND, RHS_I4, NARROW, G, 2, 2, 4>(m, stream);
+      return launch_staged<KIND, RHS_I4, NARROW, G, 2, 2, 2>(m, stream);
+    case 3:
+      *name = "mmt4d_mfma_128x64";
+      if constexpr (!RHS_I4) return launch_direct<KIND, RHS_I4, NARROW, G, 2, 1, 8>(m, stream);
+      [[fallthrough]];
+    default:
+      *name = "mmt4d_mfma_64x64";
+      if constexpr (!RHS_I4) {
+        if (direct) return launch_direct<KIND, RHS_I4, NARROW, G, 1, 1, 8>(m, stream);
+      }
+      return launch_staged<KIND, RHS_I4, NARROW, G, 1, 1, 2>(m, stream);
   }
-  if (tiles(128, 128) >= 128) {
-    *name = "mmt4d_mfma_128x128";
-    if (direct) return launch_direct<KIND, RHS_I4, NARROW, G, 2, 2, 4>(m, stream);
-    return launch_staged<KIND, RHS_I4, NARROW, G, 2, 2, 2>(m, stream);
-  }
-  *name = "mmt4d_mfma_64x64";
-  if constexpr (!RHS_I4) {
-    if (direct) return launch_direct<KIND, RHS_I4, NARROW, G, 1, 1, 8>(m, stream);
-  }
-  return launch_staged<KIND, RHS_I4, NARROW, G, 1, 1, 2>(m, stream);
 }
 
 }  // namespace

@@ -128,3 +128,13 @@ def test_float_types_ragged_256(gpu_lib, flags, M0, N0, K0, K):
 def test_s8s4s32_ragged(gpu_lib, M, N, expect):
     run_case(gpu_lib, abi.MMT4D_TYPE_S8S4S32, M, N, 6, 16, 16, 32, expect, accumulate=True, rhs_pad=64, offsets=(16, 64, 4), seed=M)
     run_case(gpu_lib, abi.MMT4D_TYPE_S8S4S32, M, N, 5, 16, 16, 16, expect, seed=N)   # 8-byte rhs pieces: staged kernel
+
+
+# The two oblong block tiles, picked for tall-and-narrow problems (few lhs rows against many rhs rows).
+@pytest.mark.parametrize("flags,M0,N0,K0,K", [(abi.MMT4D_TYPE_S8S8S32, 4, 8, 4, 32), (abi.MMT4D_TYPE_S8S8S32, 4, 16, 16, 12),
+                                              (abi.MMT4D_TYPE_F16F16F32, 4, 16, 16, 6), (abi.MMT4D_TYPE_BF16BF16F32, 4, 16, 8, 12),
+                                              (abi.MMT4D_TYPE_F32F32F32, 4, 16, 4, 8)])
+def test_oblong_tiles_ragged(gpu_lib, flags, M0, N0, K0, K):
+    n_cols = 14300 // N0 * N0
+    run_case(gpu_lib, flags, 500 // M0, n_cols // N0, K, M0, N0, K0, "mmt4d_mfma_256x128", accumulate=True, out_pad=8, seed=K)
+    run_case(gpu_lib, flags, 120 // M0, n_cols // N0, K, M0, N0, K0, "mmt4d_mfma_128x64", seed=K + 1)
