@@ -59,8 +59,10 @@ bool make_plan(const Mmt4dArgs& a, bool probe_only, Plan* plan) {
     gather = 16;
   } else if (lhs_rb >= 16 && lhs_rb <= 64) {
     gather = 16;
-  } else if (lhs_rb == 4) {
-    gather = 4;
+  } else if (lhs_rb == 4 || ((lhs_rb == 2 || lhs_rb == 8) && !narrow)) {
+    // 2 and 8 (e.g. the x86-64 int8 16x16x2 and f16 16x16x1 tiles, the Arm int8
+    // 8x8x8 tiles) run on the direct-to-LDS kernel only: see below.
+    gather = lhs_rb;
   } else {
     return false;
   }
@@ -71,7 +73,7 @@ bool make_plan(const Mmt4dArgs& a, bool probe_only, Plan* plan) {
   if (probe_only) return true;
 
   // Alignment of every vector access the kernel makes.
-  const int lhs_align = gather == 16 ? 16 : 4;
+  const int lhs_align = gather == 4 ? 4 : 16;
   const int rhs_align = i4 ? 8 : lhs_align;
   const int64_t lhs_stride_bytes = a.lhs_stride0 * elem_bytes;
   const int64_t rhs_stride_bytes = i4 ? a.rhs_stride0 / 2 : a.rhs_stride0 * elem_bytes;
@@ -98,6 +100,7 @@ bool make_plan(const Mmt4dArgs& a, bool probe_only, Plan* plan) {
   m.log2_lhs_rb = llrb; m.log2_rhs_rb = lrrb;
   m.chunks = (int32_t)(((int64_t)a.K * lhs_rb + 63) / 64);
   m.accumulate = (a.flags & IREE_UK_FLAG_MMT4D_ACCUMULATE) ? 1 : 0;
+  if ((gather == 2 || gather == 8) && !mfma_direct_covers(m, gather, i4)) return false;
   return true;
 }
 

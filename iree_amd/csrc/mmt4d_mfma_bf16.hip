@@ -9,8 +9,12 @@ hipError_t launch_mfma_bf16(const MfmaArgs& m, int gather, bool narrow, hipStrea
   if (narrow)
     return gather == 16 ? launch_variant<kBF16, false, 16, true>(m, stream, name)
                         : launch_variant<kBF16, false, 4, true>(m, stream, name);
-  return gather == 16 ? launch_variant<kBF16, false, 16, false>(m, stream, name)
-                      : launch_variant<kBF16, false, 4, false>(m, stream, name);
+  switch (gather) {
+    case 16: return launch_variant<kBF16, false, 16, false>(m, stream, name);
+    case 8: return launch_variant<kBF16, false, 8, false>(m, stream, name);
+    case 4: return launch_variant<kBF16, false, 4, false>(m, stream, name);
+    default: return launch_variant<kBF16, false, 2, false>(m, stream, name);
+  }
 }
 
 }  // namespace uk

@@ -6,8 +6,11 @@
 namespace uk {
 
 hipError_t launch_mfma_f32(const MfmaArgs& m, int gather, hipStream_t stream, const char** name) {
-  return gather == 16 ? launch_variant<kF32, false, 16, false>(m, stream, name)
-                      : launch_variant<kF32, false, 4, false>(m, stream, name);
+  switch (gather) {
+    case 16: return launch_variant<kF32, false, 16, false>(m, stream, name);
+    case 8: return launch_variant<kF32, false, 8, false>(m, stream, name);
+    default: return launch_variant<kF32, false, 4, false>(m, stream, name);
+  }
 }
 
 }  // namespace uk

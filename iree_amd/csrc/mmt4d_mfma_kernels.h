@@ -73,6 +73,10 @@ hipError_t launch_mfma_f16(const MfmaArgs& m, int gather, bool narrow, hipStream
 hipError_t launch_mfma_bf16(const MfmaArgs& m, int gather, bool narrow, hipStream_t stream, const char** name);
 hipError_t launch_mfma_f32(const MfmaArgs& m, int gather, hipStream_t stream, const char** name);
 
+// Whether the direct-to-LDS kernel covers the problem with row pieces of
+// `gather` bytes (2 and 8 have no other MFMA kernel).
+bool mfma_direct_covers(const MfmaArgs& m, int gather, bool rhs_i4);
+
 #ifdef UK_MFMA_KERNEL_BODIES
 namespace {
 
@@ -580,12 +584,17 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   //     every group of 16 lanes reads 256 contiguous bytes: no bank conflicts.
   //     (With an int4 rhs the lhs keeps the older arrangement: slot p holds row
   //     p & 31, column slot (p >> 5) & 3, read at slot 128*f + 64*kk + lane.)
-  //   G == 4: slot 64*m + l holds rows 4*g .. 4*g + 3 (g = l & 7) of fragment
-  //     m >> 1 at k step 8*(m & 1) + 4*h + d of the chunk (h = (l >> 3) & 1,
-  //     d = l >> 4). Dword 64*(8*f + 4*kk + d) + 32*h + r of the operand is then
-  //     row r of fragment f at that k step: the MFMA operand of lane 32*h + r
-  //     for K-step kk is dwords d = 0..3, each read linear in the lane number.
-  //     K is permuted inside a chunk, identically for lhs and rhs.
+  //   G == 2, 4, 8 (bytes of a row piece; R = 16 / G rows share 16 contiguous
+  //     bytes, a chunk is 64 / G k steps): slot 64*m + l holds rows R*g ..
+  //     R*g + R - 1 (g = l % (2*G)) of fragment m >> 1 at k step
+  //     (32/G)*(m & 1) + (16/G)*h + d of the chunk (h = (l / (2*G)) & 1,
+  //     d = l / (4*G)). The G-byte element number 64*((2*f + kk)*(16/G) + d) +
+  //     32*h + r of the operand is then row r of fragment f at that k step: the
+  //     MFMA operand of lane 32*h + r for K-step kk is elements d = 0 .. 16/G - 1,
+  //     each read linear in the lane number (4-byte pieces: two paired dword
+  //     reads; 8-byte: two 64-bit reads; 2-byte: eight 16-bit reads, which
+  //     makes those layouts LDS-instruction bound). K is permuted inside a
+  //     chunk, identically for lhs and rhs.
   //   int4 rhs: slot 64*f + 32*h + r holds nibbles 32*h .. 32*h + 31 of row r of
   //     fragment f: lane 32*h + r reads that slot once per chunk and widens its
   //     first 8 bytes for K-step 0, its last 8 for K-step 1. The lhs columns are
@@ -619,19 +628,20 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
                             ((16 * c) >> a.log2_rhs_rb) * rhs_kstep + ((16 * c) & (a.rhs_rb - 1)));
     }
   } else {
-    const int g = lane & 7, k1 = 4 * ((lane >> 3) & 1) + (lane >> 4);
+    constexpr int R = 16 / G;  // rows per 16-byte piece
+    const int g = lane % (2 * G), k1 = (16 / G) * ((lane / (2 * G)) & 1) + lane / (4 * G);
 #pragma unroll
     for (int t = 0; t < A_LOADS; ++t)
-      a_off[t] = (uint32_t)(row_offset(first_row + 32 * (2 * t + (wave >> 1)) + 4 * g, total_rows - 4, first_row,
+      a_off[t] = (uint32_t)(row_offset(first_row + 32 * (2 * t + (wave >> 1)) + R * g, total_rows - R, first_row,
                                        a.log2_M0, a.lhs_stride_bytes, a.lhs_rb) + k1 * lhs_kstep);
 #pragma unroll
     for (int t = 0; t < B_LOADS; ++t)
-      b_off[t] = (uint32_t)(row_offset(first_col + 32 * (2 * t + (wave >> 1)) + 4 * g, total_cols - 4, first_col,
+      b_off[t] = (uint32_t)(row_offset(first_col + 32 * (2 * t + (wave >> 1)) + R * g, total_cols - R, first_col,
                                        a.log2_N0, a.rhs_stride_bytes, a.rhs_rb) + k1 * rhs_kstep);
   }
-  // G == 4: this wavefront's loads all belong to K-step wave & 1.
-  const int64_t lhs_wave_bytes = G == 4 ? 8 * (wave & 1) * lhs_kstep : 0;
-  const int64_t rhs_wave_bytes = G == 4 ? 8 * (wave & 1) * rhs_kstep : 0;
+  // G < 16: this wavefront's loads all belong to K-step wave & 1.
+  const int64_t lhs_wave_bytes = G < 16 ? (32 / G) * (wave & 1) * lhs_kstep : 0;
+  const int64_t rhs_wave_bytes = G < 16 ? (32 / G) * (wave & 1) * rhs_kstep : 0;
 
   acc_t acc[AM][BN];
 #pragma unroll
@@ -662,6 +672,20 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   };
 
   uint4 pa[AM][2], pb[BN][2], qa[AM][2], qb[BN][2];
+  // G < 16: dword `part` (0..3) of a lane's operand for one (fragment, K-step),
+  // whose first element is at `first` (already including the lane's offset):
+  // the elements are 64*G bytes apart.
+  auto gather_dword = [](const uint8_t* first, int part) -> uint32_t {
+    if constexpr (G == 2) {
+      const uint32_t lo = *(const uint16_t*)(first + (2 * part) * 128);
+      const uint32_t hi = *(const uint16_t*)(first + (2 * part + 1) * 128);
+      return lo | (hi << 16);
+    } else if constexpr (G == 4) {
+      return *(const uint32_t*)(first + part * 256);
+    } else {
+      return *(const uint32_t*)(first + (part >> 1) * 512 + 4 * (part & 1));
+    }
+  };
   // Fragment f of an operand at 16-byte slot `operand` of the ring, K-step kk.
   auto read_frag = [&](int operand, int f, int kk) -> uint4 {
     if (RHS_I4 && operand >= A_PIECES) {
@@ -672,8 +696,8 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
       if (!RHS_I4) return ring[operand + 128 * f + 32 * kk + 64 * ((lane & 31) >> 4) + 16 * (lane >> 5) + (lane & 15)];
       return ring[operand + 128 * f + 64 * kk + lane];
     } else {
-      const uint32_t* words = (const uint32_t*)(ring + operand) + 64 * (8 * f + 4 * kk) + lane;
-      return make_uint4(words[0], words[64], words[128], words[192]);
+      const uint8_t* first = (const uint8_t*)(ring + operand) + 1024 * (2 * f + kk) + G * lane;
+      return make_uint4(gather_dword(first, 0), gather_dword(first, 1), gather_dword(first, 2), gather_dword(first, 3));
     }
   };
   const int frag_a0 = wave_m * AM, frag_b0 = wave_n * BN;
@@ -696,7 +720,7 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   constexpr bool ROWS16 = G == 16 && !RHS_I4;
   const uint8_t* ring_bytes =
       (const uint8_t*)ring + (ROWS16 ? 16 * (64 * ((lane & 31) >> 4) + 16 * (lane >> 5) + (lane & 15))
-                                     : (G == 16 ? 16 : 4) * lane);
+                                     : (G == 16 ? 16 : G) * lane);
   constexpr int KK16 = ROWS16 ? 32 : 64;
 
   // One pipeline step for the chunk whose fragments are in `cur`:
@@ -715,7 +739,9 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   auto step = [&](const uint4 (*cur_a)[2], const uint4 (*cur_b)[2], uint4 (*nxt_a)[2], uint4 (*nxt_b)[2]) {
     constexpr int SUB = SubSteps<KIND>::value;
     constexpr int MFMAS = 2 * AM * BN * SUB;
-    constexpr int PARTS = G == 4 ? 2 : 1;  // LDS read instructions per fragment (after pairing)
+    // Units a fragment's LDS reads are dealt out in: a 128-bit read; two pairs of
+    // dwords; two 64-bit reads; four pairs of 16-bit reads.
+    constexpr int PARTS = G == 16 ? 1 : (G == 2 ? 4 : 2);
     // Read units, in the order the next step consumes them: per K-step the rhs
     // fragments, then the lhs fragments. An int4 rhs fragment is read once, raw,
     // for both K-steps (first), and widened after the last read has been issued.
@@ -764,9 +790,14 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
             if constexpr (G == 16) {
               dst = *(const uint4*)(src + (128 * frag + KK16 * kk) * 16);
             } else {
-              const uint32_t* words = (const uint32_t*)src + 64 * (8 * frag + 4 * kk + 2 * part);
-              if (part == 0) { dst.x = words[0]; dst.y = words[64]; }
-              else { dst.z = words[0]; dst.w = words[64]; }
+              const uint8_t* first = src + 1024 * (2 * frag + kk);
+              if constexpr (G == 2) {
+                const uint32_t w = gather_dword(first, part);
+                if (part == 0) dst.x = w; else if (part == 1) dst.y = w; else if (part == 2) dst.z = w; else dst.w = w;
+              } else {
+                if (part == 0) { dst.x = gather_dword(first, 0); dst.y = gather_dword(first, 1); }
+                else { dst.z = gather_dword(first, 2); dst.w = gather_dword(first, 3); }
+              }
             }
           }
         }
@@ -826,8 +857,9 @@ bool direct_covers(const MfmaArgs& m) {
   if (((int64_t)m.K * m.lhs_rb) % 64 != 0) return false;
   if (RHS_I4) return m.rhs_rb >= 16 && (uintptr_t)m.rhs % 16 == 0 && m.rhs_stride_bytes % 16 == 0;
   if (G == 16) return true;
-  return m.log2_M0 >= 2 && m.log2_N0 >= 2 && (uintptr_t)m.lhs % 16 == 0 && (uintptr_t)m.rhs % 16 == 0 &&
-         m.lhs_stride_bytes % 16 == 0 && m.rhs_stride_bytes % 16 == 0;
+  // 16 / G rows of one k step make up a lane's 16 bytes: tiles at least that tall.
+  return (G << m.log2_M0) >= 16 && (G << m.log2_N0) >= 16 && (uintptr_t)m.lhs % 16 == 0 &&
+         (uintptr_t)m.rhs % 16 == 0 && m.lhs_stride_bytes % 16 == 0 && m.rhs_stride_bytes % 16 == 0;
 }
 
 void set_tile_grid(MfmaArgs* m, int block_rows, int block_cols, unsigned* grid) {
@@ -861,6 +893,10 @@ hipError_t launch_direct(MfmaArgs m, hipStream_t stream) {
 // Register-staged kernel (any K, any alignment the plan admits).
 template <int KIND, bool RHS_I4, bool NARROW, int G, int AM, int BN, int MIN_BLOCKS>
 hipError_t launch_staged(MfmaArgs m, hipStream_t stream) {
+  // 2- and 8-byte row pieces exist on the direct path only; the plan does not
+  // admit problems that would need this kernel for them.
+  if constexpr (G != 16 && G != 4) return hipErrorInvalidValue;
+  else {
   unsigned grid;
   set_tile_grid(&m, 64 * AM, 64 * BN, &grid);
   // K ending inside a chunk needs the kernel variant with the zero-filling tail step.
@@ -873,6 +909,7 @@ hipError_t launch_staged(MfmaArgs m, hipStream_t stream) {
                        dim3(256), 0, stream, m);
   }
   return hipGetLastError();
+  }
 }
 
 // Picks the block tile. Larger tiles move fewer operand bytes per multiply

@@ -138,3 +138,25 @@ def test_oblong_tiles_ragged(gpu_lib, flags, M0, N0, K0, K):
     n_cols = 14300 // N0 * N0
     run_case(gpu_lib, flags, 500 // M0, n_cols // N0, K, M0, N0, K0, "mmt4d_mfma_256x128", accumulate=True, out_pad=8, seed=K)
     run_case(gpu_lib, flags, 120 // M0, n_cols // N0, K, M0, N0, K0, "mmt4d_mfma_128x64", seed=K + 1)
+
+
+# Row pieces of 2 and 8 bytes: the tile shapes the reference's CPU targets use (x86-64 int8 16x16x2 and 8x8x2,
+# f16 16x16x1; Arm int8 8x8x8, bf16 8x8x4; mmt4d_x86_64_tiles.inl, mmt4d_arm_64_tiles.inl), i.e. what a module
+# compiled for such a CPU passes in. K is a multiple of the 64-byte chunk, as the direct-to-LDS kernel needs.
+@pytest.mark.parametrize("flags,M0,N0,K0,K", [
+    (abi.MMT4D_TYPE_S8S8S32, 16, 16, 2, 96), (abi.MMT4D_TYPE_S8S8S32, 8, 8, 2, 64), (abi.MMT4D_TYPE_S8S8S32, 8, 8, 8, 24),
+    (abi.MMT4D_TYPE_S8S8S32, 2, 8, 8, 8), (abi.MMT4D_TYPE_F16F16F32, 16, 16, 1, 64), (abi.MMT4D_TYPE_F16F16F32, 8, 8, 4, 16),
+    (abi.MMT4D_TYPE_BF16BF16F32, 8, 8, 4, 24), (abi.MMT4D_TYPE_BF16BF16F32, 16, 8, 1, 96), (abi.MMT4D_TYPE_F32F32F32, 8, 8, 2, 24)])
+def test_narrow_and_8_byte_row_pieces(gpu_lib, flags, M0, N0, K0, K):
+    # 256x256 blocks, ragged in both directions, accumulating, padded output rows
+    M, N = 3608 // M0 + 1, 3704 // N0 + 1
+    run_case(gpu_lib, flags, M, N, K, M0, N0, K0, "mmt4d_mfma_256x256", accumulate=True, out_pad=16, seed=K0 + K)
+    # the smallest block tile, strided operands with offsets (all multiples of 16 bytes)
+    run_case(gpu_lib, flags, 72 // M0, 88 // N0, K, M0, N0, K0, "mmt4d_mfma_64x64", lhs_pad=32, rhs_pad=16,
+             offsets=(16, 32, 4), seed=K0)
+
+
+def test_narrow_row_pieces_fall_back_when_the_direct_kernel_cannot_run(gpu_lib):
+    # K not a multiple of the chunk, or rows not 16-byte aligned: the generic kernel, still exact.
+    run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, 9, 11, 33, 16, 16, 2, "mmt4d_generic", accumulate=True)
+    run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, 9, 11, 32, 16, 16, 2, "mmt4d_generic", lhs_pad=4)
