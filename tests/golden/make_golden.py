@@ -119,6 +119,36 @@ def main():
         print("config 3 row", row, dt, flush=True)
     out["f16f16f32_4096_16x16x16_accumulate"] = entry
 
+    # config 2: pack f32 [8191, 8190] with 16x1 tiles, the three variants of the benchmark, and unpack of the first.
+    R, Cc = 8191, 8190
+    src = synth.normal_f32(2, 0, R * Cc)
+    entry = {"seed": [2, 0]}
+    for name, flags, o0, o1 in (("tiles16x1", 0, 512, Cc), ("transpose_inner", abi.PACK_TRANSPOSE_INNER, R, 512),
+                                ("rhs_form", abi.PACK_TRANSPOSE_INNER | abi.PACK_TRANSPOSE_OUTER, 512, R)):
+        packed = np.empty(o0 * o1 * 16, dtype=np.float32)
+        p = abi.PackParams()
+        p.in_buffer, p.out_buffer = src.ctypes.data, packed.ctypes.data
+        p.in_stride0, p.in_stride1, p.out_stride0, p.out_stride1 = Cc, 1, o1 * 16, 16
+        p.in_size0, p.in_size1 = R, Cc
+        p.out_size0, p.out_size1, p.out_size2, p.out_size3 = o0, o1, 16, 1
+        p.padding_value, p.flags = 0, abi.PACK_TYPE_F32F32 | flags
+        p.cpu_data = C.cast(cpu, C.POINTER(C.c_uint64))
+        ref.ref_pack_mt(C.byref(p), THREADS)
+        entry["pack_" + name] = digest(packed)
+        if name == "tiles16x1":
+            back = np.full(R * Cc, -1.0, dtype=np.float32)
+            u = abi.UnpackParams()
+            u.in_buffer, u.out_buffer = packed.ctypes.data, back.ctypes.data
+            u.in_stride0, u.in_stride1, u.out_stride0, u.out_stride1 = Cc * 16, 16, Cc, 1
+            u.in_size0, u.in_size1, u.in_size2, u.in_size3 = 512, Cc, 16, 1
+            u.out_size0, u.out_size1, u.flags = R, Cc, abi.UNPACK_TYPE_F32F32
+            u.cpu_data = C.cast(cpu, C.POINTER(C.c_uint64))
+            ref.ref_unpack_mt(C.byref(u), THREADS)
+            entry["unpack_tiles16x1"] = digest(back)
+            entry["source"] = digest(src)
+        print("config 2", name, flush=True)
+    out["pack_unpack_f32_8191x8190"] = entry
+
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "reference_outputs.json")
     with open(path, "w") as f:
         json.dump(out, f, separators=(",", ":"))

@@ -83,6 +83,43 @@ def test_oracle_reproduces_f16_samples_bit_for_bit(oracle_lib):
     assert np.array_equal(out[np.array(g["sample_index"][0])].view(np.uint32), want.view(np.uint32))
 
 
+PACK_VARIANTS = [("tiles16x1", 0, 512, 8190), ("transpose_inner", abi.PACK_TRANSPOSE_INNER, 8191, 512),
+                 ("rhs_form", abi.PACK_TRANSPOSE_INNER | abi.PACK_TRANSPOSE_OUTER, 512, 8191)]
+
+
+def pack_params(src, dst, flags, o0, o1):
+    p = abi.PackParams()
+    p.in_buffer, p.out_buffer = src, dst
+    p.in_stride0, p.in_stride1, p.out_stride0, p.out_stride1 = 8190, 1, o1 * 16, 16
+    p.in_size0, p.in_size1 = 8191, 8190
+    p.out_size0, p.out_size1, p.out_size2, p.out_size3 = o0, o1, 16, 1
+    p.padding_value, p.flags = 0, abi.PACK_TYPE_F32F32 | flags
+    return p
+
+
+def unpack_params(src, dst):
+    u = abi.UnpackParams()
+    u.in_buffer, u.out_buffer = src, dst
+    u.in_stride0, u.in_stride1, u.out_stride0, u.out_stride1 = 8190 * 16, 16, 8190, 1
+    u.in_size0, u.in_size1, u.in_size2, u.in_size3 = 512, 8190, 16, 1
+    u.out_size0, u.out_size1, u.flags = 8191, 8190, abi.UNPACK_TYPE_F32F32
+    return u
+
+
+@pytest.mark.parametrize("name,flags,o0,o1", PACK_VARIANTS[:2])
+def test_oracle_reproduces_pack_bit_for_bit(oracle_lib, name, flags, o0, o1):
+    g = GOLDEN["pack_unpack_f32_8191x8190"]
+    src = synth.normal_f32(2, 0, 8191 * 8190)
+    assert digest(src) == g["source"]   # the generator gives the same input everywhere
+    packed = np.empty(o0 * o1 * 16, dtype=np.float32)
+    oracle_lib.oracle_pack(C.byref(pack_params(src.ctypes.data, packed.ctypes.data, flags, o0, o1)))
+    assert digest(packed) == g["pack_" + name]
+    if name == "tiles16x1":
+        back = np.full(8191 * 8190, -1.0, dtype=np.float32)
+        oracle_lib.oracle_unpack(C.byref(unpack_params(packed.ctypes.data, back.ctypes.data)))
+        assert digest(back) == g["unpack_tiles16x1"] == g["source"]
+
+
 # ---------------------------------------------------------------------------
 # the GPU library against the reference's outputs
 # ---------------------------------------------------------------------------
@@ -155,3 +192,20 @@ def test_gpu_f16_accumulate_samples_within_tolerance(gpu):
         have = got[row * N * 256:(row + 1) * N * 256][np.array(idx)]
         rms = float(np.sqrt(np.mean(ref.astype(np.float64) ** 2)))
         assert np.all(np.abs(have - ref) <= REL_TOL * np.maximum(np.abs(ref), rms)), row
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,flags,o0,o1", PACK_VARIANTS)
+def test_gpu_pack_unpack_whole_output(gpu, name, flags, o0, o1):
+    lib, torch = gpu
+    g = GOLDEN["pack_unpack_f32_8191x8190"]
+    d_src = torch.from_numpy(synth.normal_f32(2, 0, 8191 * 8190)).cuda()
+    d_packed = torch.full((o0 * o1 * 16,), float("nan"), dtype=torch.float32, device="cuda")
+    lib.iree_uk_pack_p(C.byref(pack_params(d_src.data_ptr(), d_packed.data_ptr(), flags, o0, o1)))
+    assert lib.iree_uk_mi355x_last_kernel() == b"pack_tiled"
+    assert digest(d_packed.cpu().numpy()) == g["pack_" + name]
+    if name == "tiles16x1":
+        d_back = torch.full((8191 * 8190,), -1.0, dtype=torch.float32, device="cuda")
+        lib.iree_uk_unpack_p(C.byref(unpack_params(d_packed.data_ptr(), d_back.data_ptr())))
+        assert lib.iree_uk_mi355x_last_kernel() == b"unpack_tiled"
+        assert digest(d_back.cpu().numpy()) == g["unpack_tiles16x1"]
