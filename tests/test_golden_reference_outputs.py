@@ -106,7 +106,7 @@ def unpack_params(src, dst):
     return u
 
 
-@pytest.mark.parametrize("name,flags,o0,o1", PACK_VARIANTS[:2])
+@pytest.mark.parametrize("name,flags,o0,o1", PACK_VARIANTS)
 def test_oracle_reproduces_pack_bit_for_bit(oracle_lib, name, flags, o0, o1):
     g = GOLDEN["pack_unpack_f32_8191x8190"]
     src = synth.normal_f32(2, 0, 8191 * 8190)
