@@ -559,7 +559,6 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wave_m = wave >> 1, wave_n = wave & 1;
 
-  const int32_t M0 = 1 << a.log2_M0, N0 = 1 << a.log2_N0;
   const int64_t total_rows = (int64_t)a.M << a.log2_M0;
   const int64_t total_cols = (int64_t)a.N << a.log2_N0;
   const int64_t lhs_kstep = (int64_t)a.lhs_rb << a.log2_M0;

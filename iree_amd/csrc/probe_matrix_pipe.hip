@@ -1,0 +1,145 @@
+// A measuring stick, not part of the matmul path: what the int8 matrix pipe of
+// the device sustains on given operand bytes. One workgroup of four wavefronts
+// per compute unit runs the inner loop of the 256x256 mmt4d kernel stripped to
+// its instruction mix: per step 32 independent 32x32x32 int8 MFMAs per
+// wavefront (a 4x4 grid of accumulator fragments, two K-steps), optionally
+// with the step's memory instructions (16 128-bit LDS reads that feed the next
+// step's operands, 8 loads of 1 KiB straight to LDS, one workgroup barrier).
+// There is no HBM traffic to speak of (the loads hit in cache) and no
+// prologue or epilogue, so the rate it reports is a ceiling for any kernel
+// built on these instructions.
+//
+// Why it exists: the shader clock the device sustains depends on how many
+// bits toggle in the MFMA operands. The cycle count per step is the same for
+// all-zero and for random operand bytes; the time per step is not.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#define UK_API extern "C" __attribute__((visibility("default")))
+
+namespace {
+
+typedef int v4i32 __attribute__((ext_vector_type(4)));
+typedef int v16i32 __attribute__((ext_vector_type(16)));
+
+extern __shared__ uint4 probe_lds[];
+
+constexpr int kLdsBytes = 128 * 1024;      // lower half: what the LDS reads fetch; upper half: where the loads land
+constexpr int kOperandBytesNeeded = 2 << 20;
+
+template <bool TRAFFIC>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void probe_kernel(const uint8_t* src, int32_t* sink, int steps, long long* cycles) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  v16i32 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+  // The whole LDS starts as a copy of operand bytes (1 MiB of them, a
+  // different 128 KiB per workgroup), the first operands come from there.
+  for (int i = threadIdx.x; i < kLdsBytes / 16; i += 256)
+    probe_lds[i] = ((const uint4*)src)[i + (kLdsBytes / 16) * (blockIdx.x & 7)];
+  __syncthreads();
+  uint4 cur[16], nxt[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    cur[i] = probe_lds[(i * 64 + lane) & 8191];
+    nxt[i] = probe_lds[(i * 64 + lane + 1024) & 8191];
+  }
+  const uint8_t* read_base = (const uint8_t*)probe_lds + wave * 16384 + lane * 16;
+  const uint32_t voff = lane * 16;
+  const uint8_t* load_base = src + (1 << 20) + (size_t)(blockIdx.x & 15) * 65536 + wave * 8192;
+  const long long t0 = clock64();
+  auto step = [&](uint4 (&c)[16], uint4 (&n)[16], int s) {
+#pragma unroll
+    for (int m = 0; m < 32; ++m) {
+      const int kk = m >> 4, i = (m >> 2) & 3, j = m & 3;
+      if (TRAFFIC && m == 4) {
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+      }
+      if (TRAFFIC && m >= 4 && m < 28 && (m - 4) % 3 == 0) {
+        const int t = (m - 4) / 3;
+        const uint32_t lds_off = (uint32_t)(65536 + ((s & 1) * 32 + t * 4 + wave) * 1024);
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(lds_off), "v"(voff + t * 1024), "s"(load_base)
+                     : "memory");
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (TRAFFIC && m >= 4 && m < 28) {
+        const int slot = m - 4;  // 16 reads dealt out over 24 MFMAs
+#pragma unroll
+        for (int u = slot * 16 / 24; u < (slot + 1) * 16 / 24; ++u) n[u] = *(const uint4*)(read_base + u * 1024);
+      }
+      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(v4i32, c[8 * kk + 4 + j]),
+                                                        __builtin_bit_cast(v4i32, c[8 * kk + i]), acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  for (int s = 0; s < steps; s += 2) {
+    step(cur, nxt, s);
+    step(nxt, cur, s + 1);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  const long long t1 = clock64();
+  int32_t x = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) x ^= acc[i][j][v];
+  // Keeps the accumulators alive; practically never true.
+  if (x == 0x7654321 && steps < 0) sink[0] = x;
+  if (threadIdx.x == 0 && blockIdx.x == 0) cycles[0] = t1 - t0;
+}
+
+}  // namespace
+
+UK_API int iree_uk_mi355x_probe_int8_matrix_pipe(const void* operand_bytes, long long operand_size, int memory_traffic,
+                                                 int steps, double* tera_ops_per_second, double* shader_mhz) {
+  if (operand_bytes == nullptr || operand_size < kOperandBytesNeeded || steps < 2 || (steps & 1)) {
+    return (int)hipErrorInvalidValue;
+  }
+  int device = 0, cus = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
+  if (e != hipSuccess) return (int)e;
+  long long* scratch = nullptr;  // [0]: cycles of workgroup 0; [1]: sink
+  e = hipMalloc((void**)&scratch, 64);
+  if (e != hipSuccess) return (int)e;
+  hipEvent_t begin = nullptr, end = nullptr;
+  float ms = 0.f;
+  long long cycles = 0;
+  auto kernel = memory_traffic ? probe_kernel<true> : probe_kernel<false>;
+  e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+  if (e == hipSuccess) e = hipEventCreate(&begin);
+  if (e == hipSuccess) e = hipEventCreate(&end);
+  if (e == hipSuccess) {
+    // One untimed launch (clock ramp, instruction cache), one timed.
+    for (int rep = 0; rep < 2 && e == hipSuccess; ++rep) {
+      e = hipEventRecord(begin, nullptr);
+      hipLaunchKernelGGL(kernel, dim3(cus), dim3(256), kLdsBytes, nullptr, (const uint8_t*)operand_bytes,
+                         (int32_t*)(scratch + 1), steps, scratch);
+      if (e == hipSuccess) e = hipGetLastError();
+      if (e == hipSuccess) e = hipEventRecord(end, nullptr);
+      if (e == hipSuccess) e = hipEventSynchronize(end);
+    }
+  }
+  if (e == hipSuccess) e = hipEventElapsedTime(&ms, begin, end);
+  if (e == hipSuccess) e = hipMemcpy(&cycles, scratch, sizeof(cycles), hipMemcpyDeviceToHost);
+  if (begin) (void)hipEventDestroy(begin);
+  if (end) (void)hipEventDestroy(end);
+  (void)hipFree(scratch);
+  if (e != hipSuccess) return (int)e;
+  const double ops = (double)cus * 4 * steps * 32 * (2.0 * 32 * 32 * 32);
+  if (tera_ops_per_second) *tera_ops_per_second = ops / (ms * 1e-3) / 1e12;
+  if (shader_mhz) *shader_mhz = (double)cycles / (ms * 1e3);
+  return 0;
+}
