@@ -14,9 +14,21 @@
 // kernels move bytes, so results are bit-exact by construction; padding is the
 // low bytes of padding_value (pack.h:15-24).
 //
+// With an inner transpose the tiled side's 16 contiguous bytes are 16 / E
+// consecutive ROWS of one column. For 4-byte elements that is four 32-bit LDS
+// reads per vector; for 1- and 2-byte elements it would be 16 or 8 narrow
+// reads, which makes the kernel LDS-instruction bound (3.5 TB/s for int8). Pack
+// with such elements goes through pack_transposing_kernel instead: a thread
+// loads 16 bytes from each of 4 / E consecutive rows, transposes the 4x4 bytes
+// (2x2 halfwords) blocks in registers (v_perm_b32), and writes dwords into an
+// LDS image that is already in tiled order; the tiled side then is one 128-bit
+// LDS read and one 128-bit store per vector.
+//
 // Anything this file does not cover (non power-of-two tiles, inner stride on
 // the 2-D side, unaligned tiled buffers) goes to the generic kernels.
+#include <mutex>
 #include <type_traits>
+#include <vector>
 
 #include "uk_internal.h"
 
@@ -42,6 +54,10 @@ struct TiledArgs {
   int32_t blocks1;           // blocks along dim 1
   int32_t total_blocks;
   int32_t tr_inner, tr_outer;
+  // pack_transposing_kernel only: consecutive lanes along a row before the next
+  // row group starts, and the LDS image's skew (pad_bytes inserted every
+  // 1 << log2_period bytes).
+  int32_t log2_lpr, log2_period, pad_bytes;
 };
 
 // Coordinates of an element of the tiled side within a block.
@@ -192,6 +208,16 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
         const int64_t row = row_base + r, col = col_base + (int64_t)cv * EPV;
         uint8_t* g = a.dst + (row * a.flat_stride0 + col) * E;
         if (row < a.size0 && col + EPV <= a.size1) {
+          // Whole vectors inside the matrix: written once, not read here.
+          if constexpr (W == 16) {
+            typedef int v4 __attribute__((ext_vector_type(4)));
+            __builtin_nontemporal_store(v4{(int)regs[u].vec.x, (int)regs[u].vec.y, (int)regs[u].vec.z, (int)regs[u].vec.w}, (v4*)g);
+          } else if constexpr (W == 8) {
+            typedef int v2 __attribute__((ext_vector_type(2)));
+            __builtin_nontemporal_store(v2{(int)regs[u].vec.x, (int)regs[u].vec.y}, (v2*)g);
+          } else if constexpr (W == 4) {
+            __builtin_nontemporal_store(regs[u].vec, (flat_vec_t*)g);
+          } else
           *(flat_vec_t*)g = regs[u].vec;
         } else if (row < a.size0) {
 #pragma unroll
@@ -253,6 +279,116 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
     tiled_phase();
     __syncthreads();
     flat_store_phase();
+  }
+}
+
+// Element (row, col) of a block -> its index in the block's tiled-side
+// enumeration (the inverse of tiled_coord), for an inner transpose.
+__host__ __device__ __forceinline__ int32_t tiled_index_tr_inner(const TiledArgs& a, int32_t row, int32_t col) {
+  const int32_t log2_tile = a.log2_t0 + a.log2_t1;
+  const int32_t o0l = row >> a.log2_t0, t0 = row & ((1 << a.log2_t0) - 1);
+  const int32_t o1l = col >> a.log2_t1, t1 = col & ((1 << a.log2_t1) - 1);
+  const int32_t w = (t1 << a.log2_t0) | t0;
+  if (!a.tr_outer) return (o0l << (a.log2_bc + a.log2_t0)) | (o1l << log2_tile) | w;
+  return (o1l << (a.log2_br + a.log2_t1)) | (o0l << log2_tile) | w;
+}
+
+__host__ __device__ __forceinline__ uint32_t skewed(const TiledArgs& a, uint32_t byte_offset) {
+  return byte_offset + (byte_offset >> a.log2_period) * a.pad_bytes;
+}
+
+// Unit v (of the block's kBlockBytes / (RQ * 16)) -> its first row and column:
+// 1 << log2_lpr units side by side along a row, then down all row groups, then
+// the next stretch of columns.
+__host__ __device__ __forceinline__ void transposing_unit(const TiledArgs& a, int32_t v, int rq, int ve, int32_t* row0,
+                                                          int32_t* col0) {
+  const int32_t log2_rg = a.log2_br - (rq == 4 ? 2 : 1);
+  const int32_t cg_lo = v & ((1 << a.log2_lpr) - 1), rest = v >> a.log2_lpr;
+  const int32_t rg = rest & ((1 << log2_rg) - 1), cg_hi = rest >> log2_rg;
+  *row0 = rg * rq;
+  *col0 = ((cg_hi << a.log2_lpr) | cg_lo) * ve;
+}
+
+// Pack with an inner transpose for 1- and 2-byte elements (see the top of the
+// file). Needs rows that are 4-byte aligned and tiles at least 4 / E rows tall.
+template <int E>
+__global__ __launch_bounds__(256) void pack_transposing_kernel(const TiledArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  typedef typename std::conditional<E == 1, uint8_t, uint16_t>::type elem_t;
+  constexpr int RQ = 4 / E;   // rows whose elements of one column make up a dword
+  constexpr int VE = 16 / E;  // columns per 16-byte vector
+  constexpr int UNITS = kBlockBytes / (RQ * 16) / 256;
+  constexpr int TILED_PER_THREAD = kBlockBytes / 16 / 256;
+
+  const int tid = threadIdx.x;
+  const int32_t per_xcd = (a.total_blocks + 7) >> 3;
+  const int32_t linear = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (linear >= a.total_blocks) return;
+  const int64_t block0 = linear / a.blocks1, block1 = linear % a.blocks1;
+  const int64_t row_base = block0 << a.log2_br, col_base = block1 << a.log2_bc;
+  const int64_t tile0_base = row_base >> a.log2_t0, tile1_base = col_base >> a.log2_t1;
+
+  union RowVec {
+    uint32_t dword[4];
+    elem_t elem[VE];
+  };
+  RowVec regs[UNITS][RQ];
+  int32_t row0[UNITS], col0[UNITS];
+#pragma unroll
+  for (int u = 0; u < UNITS; ++u) {
+    transposing_unit(a, tid + 256 * u, RQ, VE, &row0[u], &col0[u]);
+#pragma unroll
+    for (int j = 0; j < RQ; ++j) {
+      const int64_t row = row_base + row0[u] + j, col = col_base + col0[u];
+      const uint8_t* g = a.src + (row * a.flat_stride0 + col) * E;
+      if (row < a.size0 && col + VE <= a.size1) {
+        typedef int v4a4 __attribute__((ext_vector_type(4), aligned(4)));
+        const v4a4 t = __builtin_nontemporal_load((const v4a4*)g);
+        regs[u][j].dword[0] = t.x; regs[u][j].dword[1] = t.y; regs[u][j].dword[2] = t.z; regs[u][j].dword[3] = t.w;
+      } else {
+#pragma unroll
+        for (int i = 0; i < VE; ++i) {
+          elem_t x = (elem_t)a.padding_value;
+          if (row < a.size0 && col + i < a.size1) x = ((const elem_t*)g)[i];
+          regs[u][j].elem[i] = x;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < UNITS; ++u) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      uint32_t out[RQ];
+      if constexpr (E == 1) {
+        const uint32_t ra = regs[u][0].dword[k], rb = regs[u][1].dword[k], rc = regs[u][2].dword[k], rd = regs[u][3].dword[k];
+        const uint32_t ab_lo = __builtin_amdgcn_perm(rb, ra, 0x05010400u), ab_hi = __builtin_amdgcn_perm(rb, ra, 0x07030602u);
+        const uint32_t cd_lo = __builtin_amdgcn_perm(rd, rc, 0x05010400u), cd_hi = __builtin_amdgcn_perm(rd, rc, 0x07030602u);
+        out[0] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x05040100u);
+        out[1] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x07060302u);
+        out[2] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x05040100u);
+        out[3] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x07060302u);
+      } else {
+        const uint32_t ra = regs[u][0].dword[k], rb = regs[u][1].dword[k];
+        out[0] = __builtin_amdgcn_perm(rb, ra, 0x05040100u);
+        out[1] = __builtin_amdgcn_perm(rb, ra, 0x07060302u);
+      }
+#pragma unroll
+      for (int i = 0; i < RQ; ++i) {
+        const int32_t e = tiled_index_tr_inner(a, row0[u], col0[u] + RQ * k + i);
+        *(uint32_t*)(lds + skewed(a, (uint32_t)e * E)) = out[i];
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < TILED_PER_THREAD; ++u) {
+    const int32_t q = tid + 256 * u;
+    const TiledCoord c = tiled_coord(a, q * VE, tile0_base, tile1_base);
+    if (!c.in_range) continue;
+    typedef int v4 __attribute__((ext_vector_type(4)));
+    const v4 vec = *(const v4*)(lds + skewed(a, (uint32_t)q * 16));
+    __builtin_nontemporal_store(vec, (v4*)(a.dst + c.global_elem * E));
   }
 }
 
@@ -415,6 +551,77 @@ bool make_plan(const uint8_t* flat, const uint8_t* tiled, int64_t flat_stride0, 
   return plan->lds_bytes <= 49152;
 }
 
+// Lane arrangement and LDS skew for pack_transposing_kernel: the combination
+// with the fewest bank conflicts among the dword writes of one wavefront
+// (32 lanes per pass over 32 banks), found by trying them on the host. The
+// search takes about a millisecond, so results are kept per block geometry.
+struct TransposingChoice {
+  uint32_t key;
+  int32_t log2_lpr, log2_period, pad_bytes;
+};
+
+void choose_transposing(TiledArgs* a, int elem_bytes) {
+  static std::mutex mutex;
+  static std::vector<TransposingChoice> known;
+  const uint32_t key = (uint32_t)elem_bytes | (uint32_t)a->log2_t0 << 4 | (uint32_t)a->log2_t1 << 8 |
+                       (uint32_t)a->log2_br << 12 | (uint32_t)a->log2_bc << 17 | (uint32_t)a->tr_outer << 22;
+  std::lock_guard<std::mutex> lock(mutex);
+  for (const TransposingChoice& c : known) {
+    if (c.key == key) {
+      a->log2_lpr = c.log2_lpr; a->log2_period = c.log2_period; a->pad_bytes = c.pad_bytes;
+      return;
+    }
+  }
+  const int rq = 4 / elem_bytes, ve = 16 / elem_bytes;
+  const int log2_cg = a->log2_bc + (elem_bytes == 2 ? 1 : 0) - 4;
+  TransposingChoice best{key, 0, 14, 0};
+  long best_cost = -1;
+  TiledArgs t = *a;
+  for (t.log2_lpr = log2_cg < 2 ? log2_cg : 2; t.log2_lpr <= log2_cg; ++t.log2_lpr) {
+    for (t.log2_period = 6; t.log2_period <= 14; ++t.log2_period) {
+      for (t.pad_bytes = 0; t.pad_bytes <= 64; t.pad_bytes += 16) {
+        if (t.log2_period == 14 && t.pad_bytes) break;  // one period: padding changes nothing
+        long cost = 0;
+        for (int i = 0; i < ve; ++i) {
+          for (int half = 0; half < 2; ++half) {
+            int hits[32] = {0};
+            int worst = 0;
+            for (int lane = 32 * half; lane < 32 * half + 32; ++lane) {
+              int32_t row0, col0;
+              transposing_unit(t, lane, rq, ve, &row0, &col0);
+              const uint32_t addr = skewed(t, (uint32_t)tiled_index_tr_inner(t, row0, col0 + i) * elem_bytes);
+              const int h = ++hits[(addr >> 2) & 31];
+              worst = h > worst ? h : worst;
+            }
+            cost += worst;
+          }
+        }
+        // Fewest conflicts; then the longest contiguous stretch of a row per
+        // load instruction; then the least padding.
+        const long ranked = cost * 1000 - t.log2_lpr * 10 + t.pad_bytes / 16;
+        if (best_cost < 0 || ranked < best_cost) {
+          best_cost = ranked;
+          best.log2_lpr = t.log2_lpr; best.log2_period = t.log2_period; best.pad_bytes = t.pad_bytes;
+        }
+      }
+    }
+  }
+  known.push_back(best);
+  a->log2_lpr = best.log2_lpr; a->log2_period = best.log2_period; a->pad_bytes = best.pad_bytes;
+}
+
+// Whether pack_transposing_kernel takes the planned call; sets it up if so.
+bool plan_transposing(Plan* p) {
+  TiledArgs& a = p->args;
+  const int E = p->elem_bytes;
+  if (!a.tr_inner || E > 2 || p->flat_vec_bytes != 16) return false;
+  const int log2_rq = E == 1 ? 2 : 1;
+  if (a.log2_t0 < log2_rq || a.log2_bc + (E == 2 ? 1 : 0) < 4) return false;
+  choose_transposing(&a, E);
+  p->lds_bytes = skewed(a, kBlockBytes - 16) + 16;
+  return true;
+}
+
 template <int E, int W, bool UNPACK>
 hipError_t launch_pw(const Plan& p, hipStream_t stream) {
   const dim3 grid(p.grid), block(256);
@@ -473,6 +680,15 @@ hipError_t launch_pack(const PackArgs& a, hipStream_t stream, const char** name)
   plan.args.src = a.in;
   plan.args.dst = a.out;
   plan.args.padding_value = a.padding_value;
+  if (plan_transposing(&plan)) {
+    *name = "pack_transposing";
+    if (plan.elem_bytes == 1) {
+      hipLaunchKernelGGL(pack_transposing_kernel<1>, dim3(plan.grid), dim3(256), plan.lds_bytes, stream, plan.args);
+    } else {
+      hipLaunchKernelGGL(pack_transposing_kernel<2>, dim3(plan.grid), dim3(256), plan.lds_bytes, stream, plan.args);
+    }
+    return hipGetLastError();
+  }
   *name = "pack_tiled";
   return launch_plan<false>(plan, stream);
 }
