@@ -283,6 +283,46 @@ def _also(torch, lib, abi, synth, steps, warmup):
     timed_pair("unpack_f32_512x8190x16x1_to_8191x8190", unpack_params, 2 * R * Cc * 4)
     torch.cuda.synchronize()
     res["pack_unpack_round_trip_bit_exact"] = bool(all(torch.equal(src[i], back[i]) for i in range(2)))
+    del src, packed, back
+
+    # int8 operands of a 16384^3 matmul into the layouts of the 16x16x64 tile:
+    # lhs [16384, 16384] -> [1024, 256, 16, 64]; rhs [K=16384, N=16384] ->
+    # [1024, 256, 16, 64] with both transposes (n-tile outermost, k innermost).
+    # Three buffer sets (each 537 MB) rotated.
+    n16 = 16384
+    isrc = [torch.from_numpy(synth.uniform_int8(8, i, n16 * n16)).cuda() for i in range(3)]
+    idst = [torch.empty(n16 * n16, dtype=torch.int8, device="cuda") for _ in range(3)]
+
+    def pack_i8(i, flags, s2, s3):
+        p = abi.PackParams()
+        p.in_buffer, p.out_buffer = isrc[i].data_ptr(), idst[i].data_ptr()
+        p.in_stride0, p.in_stride1 = n16, 1
+        p.out_size0, p.out_size1, p.out_size2, p.out_size3 = 1024, 256, s2, s3
+        p.out_stride0, p.out_stride1 = 256 * s2 * s3, s2 * s3
+        p.in_size0, p.in_size1 = n16, n16
+        p.padding_value = 0
+        p.flags = abi.PACK_TYPE_I8I8 | flags
+        return p
+
+    def timed_three(name, flags):
+        ps = [pack_i8(i, flags, 16, 64) for i in range(3)]
+        state = {"i": 0}
+
+        def step():
+            lib.iree_uk_pack_p(C.byref(ps[state["i"] % 3]))
+            state["i"] += 1
+        ms, _ = _time_launches(torch, step, max(steps, 6), warmup)
+        res[name] = {"kernel": lib.iree_uk_mi355x_last_kernel().decode(), "ms": round(ms, 5),
+                     "value": round(2.0 * n16 * n16 / ms / 1e6, 1), "unit": "GB/s",
+                     "frac_of_peak": round(2.0 * n16 * n16 / ms / 1e6 / PEAK_HBM_GBS, 4)}
+    timed_three("pack_i8_16384x16384_lhs_to_1024x256x16x64", 0)
+    timed_three("pack_i8_16384x16384_rhs_transpose_both_to_1024x256x16x64",
+                abi.PACK_TRANSPOSE_INNER | abi.PACK_TRANSPOSE_OUTER)
+    # The rhs result against the same permutation done by torch.
+    want = isrc[0].view(256, 64, 1024, 16).permute(2, 0, 3, 1).contiguous().view(-1)
+    lib.iree_uk_pack_p(C.byref(pack_i8(0, abi.PACK_TRANSPOSE_INNER | abi.PACK_TRANSPOSE_OUTER, 16, 64)))
+    torch.cuda.synchronize()
+    res["pack_i8_rhs_layout_bit_exact"] = bool(torch.equal(want, idst[0]))
     return res
 
 
