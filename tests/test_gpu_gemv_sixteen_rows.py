@@ -1,0 +1,62 @@
+"""GPU parity for the skinny-lhs kernel (mmt4d_gemv.hip) on one 16-row lhs tile,
+against the oracle restatement of the generic tile functions
+(mmt4d_tile_generic.c:54-78 int8, :199-225 f16, :289-315 bf16): every row-piece
+size it takes, odd rhs tile counts, K shares that are not a multiple of the
+unrolling, K that does not end on a 64-byte step, accumulate, strided rhs.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from iree_amd import abi, synth
+from test_gpu_configs import assert_float_close, gpu_lib, mm_params  # noqa: F401
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # flags, N, K, K0, expected kernel
+    (abi.MMT4D_TYPE_BF16BF16F32, 37, 512, 8, b"mmt4d_gemv"),     # rb 16, N % 4 != 0
+    (abi.MMT4D_TYPE_BF16BF16F32, 64, 4 * 17, 8, b"mmt4d_gemv"),  # 17 K-steps: shares of 5, 5, 5, 2
+    (abi.MMT4D_TYPE_F16F16F32, 50, 256, 16, b"mmt4d_gemv"),      # rb 32
+    (abi.MMT4D_TYPE_S8S8S32, 41, 64, 64, b"mmt4d_gemv"),         # rb 64
+    (abi.MMT4D_TYPE_S8S8S32, 29, 128, 32, b"mmt4d_gemv"),        # rb 32, int8
+    (abi.MMT4D_TYPE_S8S8S32, 33, 260, 16, b"mmt4d_gemv"),        # rb 16, 65 K-steps
+    (abi.MMT4D_TYPE_BF16BF16F32, 20, 1026, 8, b"mmt4d_gemv"),        # K does not end on a K-step
+    (abi.MMT4D_TYPE_BF16BF16F32, 24, 8200, 8, b"mmt4d_gemv"),        # long K
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "t%x_N%d_K%d_K0%d" % (c[0], c[1], c[2], c[3]))
+@pytest.mark.parametrize("acc", [0, abi.MMT4D_ACCUMULATE])
+def test_sixteen_row_lhs(gpu_lib, oracle_lib, case, acc):
+    flags, N, K, K0, kernel = case
+    M0 = N0 = 16
+    flags |= acc
+    rhs_stride = K * N0 * K0 + 64  # elements; a gap between rhs panels
+    if (flags & 0xFF) == abi.MMT4D_TYPE_S8S8S32:
+        lhs = synth.uniform_int8(41, 0, K * M0 * K0)
+        rhs = synth.uniform_int8(41, 1, N * rhs_stride)
+        init = (synth.uniform_int8(41, 2, N * M0 * N0).astype(np.int32)) * 1000
+    else:
+        to_bits = synth.f16_bits if (flags & 0xFF) == abi.MMT4D_TYPE_F16F16F32 else synth.bf16_bits
+        lhs = to_bits(synth.normal_f32(41, 0, K * M0 * K0, 1.0))
+        rhs = to_bits(synth.normal_f32(41, 1, N * rhs_stride, 0.05))
+        init = synth.normal_f32(41, 2, N * M0 * N0, 1.0)
+    want = init.copy()
+    p = mm_params(lhs.ctypes.data, rhs.ctypes.data, want.ctypes.data, 1, N, K, M0, N0, K0,
+                  flags | abi.MMT4D_ALLOW_GENERIC_FALLBACK)
+    p.rhs_stride0 = rhs_stride
+    oracle_lib.oracle_mmt4d_mt(C.byref(p), 8)
+    as_dev = lambda x: torch.from_numpy(x.view(np.int16) if x.dtype == np.uint16 else x).cuda()
+    d_l, d_r, d_o = as_dev(lhs), as_dev(rhs), as_dev(init.copy())
+    q = mm_params(d_l.data_ptr(), d_r.data_ptr(), d_o.data_ptr(), 1, N, K, M0, N0, K0, flags)
+    q.rhs_stride0 = rhs_stride
+    gpu_lib.iree_uk_mmt4d_p(C.byref(q))
+    assert gpu_lib.iree_uk_mi355x_last_kernel() == kernel
+    got = d_o.cpu().numpy()
+    if want.dtype == np.int32:
+        assert np.array_equal(got, want)
+    else:
+        assert_float_close(got, want, "16-row lhs N=%d K=%d K0=%d" % (N, K, K0))
