@@ -643,6 +643,12 @@ bool make_plan(const uint8_t* flat, const uint8_t* tiled, int64_t flat_stride0, 
     // shorten the contiguous runs on the tiled side).
     bc = 1024 / E;
     while (bc * E > 256 && kBlockBytes / (bc * E) < T0) bc /= 2;
+    // The runs on the tiled side (rows x tile width) must be whole cache lines:
+    // with narrow tiles a 16-row block has runs of 16 to 64 bytes, and each
+    // 128-byte line is then written in pieces by several blocks (int8 8x2
+    // tiles: 1.8 TB/s; with 64 rows x 256 bytes instead 4.7 TB/s). Longer runs
+    // than a line at the price of shorter row pieces measured slower again.
+    while (bc * E > 128 && (kBlockBytes / (bc * E)) * T1 * E < 128) bc /= 2;
     if (bc < T1) bc = T1;
     br = kBlockBytes / (bc * E);
   }
