@@ -13,7 +13,8 @@
 // and it keeps the VALU out of the inner loop.
 //
 // Covers s8s8s32, f16f16f32 and bf16bf16f32 with N0 = 16 and 16, 32 or 64
-// bytes per (k, row) piece.
+// bytes per (k, row) piece, and s8s4s32 (int4 weights) with N0 = 16 and
+// K0 = 32 or 64 (mmt4d_gemv_i4_kernel below).
 #include "uk_internal.h"
 
 namespace uk {
@@ -24,7 +25,7 @@ typedef float v4f32 __attribute__((ext_vector_type(4)));
 typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
 typedef __bf16 v8bf16 __attribute__((ext_vector_type(8)));
 
-enum Kind { kI8 = 0, kF16 = 1, kBF16 = 2 };
+enum Kind { kI8 = 0, kF16 = 1, kBF16 = 2, kI8I4 = 3 };
 
 struct GemvArgs {
   const uint8_t* lhs;
@@ -148,6 +149,116 @@ __global__ __launch_bounds__(64 * kWaves) void mmt4d_gemv_kernel(const GemvArgs 
   }
 }
 
+// int8 values equal to 16x the signed nibbles of 8 bytes, in element order
+// (element 2b in the low nibble of byte b, mmt4d_tile_generic.c:35-45): even
+// and odd elements are isolated in the high nibbles of two dwords whose bytes
+// are then interleaved. Products with these are 16x too large and exact.
+__device__ __forceinline__ uint4 widen_i4_times16(uint32_t lo, uint32_t hi) {
+  const uint32_t even0 = (lo << 4) & 0xF0F0F0F0u, odd0 = lo & 0xF0F0F0F0u;
+  const uint32_t even1 = (hi << 4) & 0xF0F0F0F0u, odd1 = hi & 0xF0F0F0F0u;
+  uint4 r;
+  r.x = __builtin_amdgcn_perm(odd0, even0, 0x05010400u);
+  r.y = __builtin_amdgcn_perm(odd0, even0, 0x07030602u);
+  r.z = __builtin_amdgcn_perm(odd1, even1, 0x05010400u);
+  r.w = __builtin_amdgcn_perm(odd1, even1, 0x07030602u);
+  return r;
+}
+
+// s8s4s32 for a skinny lhs: the int4 rhs streams at half a byte per weight.
+// One step covers 128 values of K. Lane l (row l & 15, g = l >> 4) loads the 16
+// bytes = 32 nibbles of its rhs row at K values 32*g .. 32*g + 31 of the step
+// (for K0 = 32 that is row l & 15 of k step g: the wavefront reads 1 KiB of
+// contiguous rhs per load instruction), widens them to two int8 operands, and
+// multiplies each with the matching 16 bytes of the lhs (the MFMA sums over K in
+// whatever order the two operands agree on). Accumulators carry 16x the result
+// until the end; K * K0 < 131072 keeps that inside int32.
+// TN rhs tiles per workgroup share each lhs operand: with 16 lhs rows the lhs
+// is twice the bytes of one rhs tile per step (int8 against int4), all of it
+// through L2 for every workgroup.
+template <int TN, int UNROLL, int kWaves>
+__global__ __launch_bounds__(64 * kWaves) void mmt4d_gemv_i4_kernel(const GemvArgs a) {
+  __shared__ v4i32 partial[kWaves][TN][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int row = lane & 15, g = lane >> 4;
+  const int32_t M0 = 1 << a.log2_M0;
+  const int32_t lhs_rows = a.M << a.log2_M0;  // <= 16
+  // a.rb / a.log2_rb describe the lhs row piece (K0 bytes); the rhs piece is half of it.
+  const int32_t rhs_rb = a.rb >> 1, log2_rhs_rb = a.log2_rb - 1;
+  const int64_t lhs_kstep = (int64_t)a.rb << a.log2_M0;
+  const bool lhs_valid = row < lhs_rows;
+  const uint8_t* lhs_lane = a.lhs + (int64_t)(row >> a.log2_M0) * a.lhs_stride_bytes +
+                            (int64_t)(row & (M0 - 1)) * a.rb + ((32 * g) >> a.log2_rb) * lhs_kstep +
+                            ((32 * g) & (a.rb - 1));
+  const int64_t lhs_step_bytes = (int64_t)128 << a.log2_M0;
+  const int64_t tile0 = (int64_t)blockIdx.x * TN;
+  const uint8_t* rhs_lane[TN];
+#pragma unroll
+  for (int t = 0; t < TN; ++t) {
+    const int64_t tile = tile0 + t < a.N ? tile0 + t : a.N - 1;  // clamp: computed, not stored
+    rhs_lane[t] = a.rhs + tile * a.rhs_stride_bytes + (int64_t)row * rhs_rb +
+                  ((16 * g) >> log2_rhs_rb) * ((int64_t)rhs_rb * 16) + ((16 * g) & (rhs_rb - 1));
+  }
+
+  const int32_t per_wave = (a.steps + kWaves - 1) / kWaves;
+  const int32_t s_begin = wave * per_wave;
+  const int32_t s_end = min(s_begin + per_wave, a.steps);
+
+  v4i32 acc[TN];
+#pragma unroll
+  for (int t = 0; t < TN; ++t) acc[t] = v4i32{0, 0, 0, 0};
+  auto multiply = [&](int t, uint4 r, uint4 l0, uint4 l1) {
+    acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i32, widen_i4_times16(r.x, r.y)),
+                                                   __builtin_bit_cast(v4i32, l0), acc[t], 0, 0, 0);
+    acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i32, widen_i4_times16(r.z, r.w)),
+                                                   __builtin_bit_cast(v4i32, l1), acc[t], 0, 0, 0);
+  };
+  int32_t s = s_begin;
+  for (; s + UNROLL <= s_end; s += UNROLL) {
+    uint4 r[UNROLL][TN], l0[UNROLL], l1[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+#pragma unroll
+      for (int t = 0; t < TN; ++t)
+        r[u][t] = __builtin_bit_cast(uint4, __builtin_nontemporal_load((const v4i32*)(rhs_lane[t] + (int64_t)(s + u) * 1024)));
+      l0[u] = l1[u] = make_uint4(0, 0, 0, 0);
+      if (lhs_valid) {
+        l0[u] = *(const uint4*)(lhs_lane + (s + u) * lhs_step_bytes);
+        l1[u] = *(const uint4*)(lhs_lane + (s + u) * lhs_step_bytes + 16);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+      for (int t = 0; t < TN; ++t) multiply(t, r[u][t], l0[u], l1[u]);
+  }
+  for (; s < s_end; ++s) {
+    uint4 l0 = make_uint4(0, 0, 0, 0), l1 = l0;
+    if (lhs_valid) {
+      l0 = *(const uint4*)(lhs_lane + s * lhs_step_bytes);
+      l1 = *(const uint4*)(lhs_lane + s * lhs_step_bytes + 16);
+    }
+#pragma unroll
+    for (int t = 0; t < TN; ++t) multiply(t, *(const uint4*)(rhs_lane[t] + (int64_t)s * 1024), l0, l1);
+  }
+
+#pragma unroll
+  for (int t = 0; t < TN; ++t) partial[wave][t][lane] = acc[t];
+  __syncthreads();
+  if (wave != 0 || !lhs_valid) return;
+#pragma unroll
+  for (int t = 0; t < TN; ++t) {
+    if (tile0 + t >= a.N) continue;
+    v4i32 v = partial[0][t][lane];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) v += partial[w][t][lane];
+    v = v4i32{v.x >> 4, v.y >> 4, v.z >> 4, v.w >> 4};
+    v4i32* dst = (v4i32*)(a.out + 4 * ((int64_t)(row >> a.log2_M0) * a.out_stride0 + (tile0 + t) * ((int64_t)M0 * 16) +
+                                       (int64_t)(row & (M0 - 1)) * 16 + 4 * g));
+    if (a.accumulate) v += *dst;
+    *dst = v;
+  }
+}
+
 int log2_exact(int64_t v) {
   if (v <= 0 || (v & (v - 1))) return -1;
   int l = 0;
@@ -157,8 +268,10 @@ int log2_exact(int64_t v) {
 
 bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, GemvArgs* g) {
   int elem_bytes;
+  bool i4 = false;
   switch (a.flags & IREE_UK_FLAG_MMT4D_TYPE_MASK) {
     case IREE_UK_FLAG_MMT4D_TYPE_S8S8S32: *kind = kI8; elem_bytes = 1; break;
+    case IREE_UK_FLAG_MMT4D_TYPE_S8S4S32: *kind = kI8I4; elem_bytes = 1; i4 = true; break;
     case IREE_UK_FLAG_MMT4D_TYPE_F16F16F32: *kind = kF16; elem_bytes = 2; break;
     case IREE_UK_FLAG_MMT4D_TYPE_BF16BF16F32: *kind = kBF16; elem_bytes = 2; break;
     default: return false;
@@ -167,12 +280,15 @@ bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, GemvArgs* g) {
   const int rb = a.K0 * elem_bytes;
   if (lm0 < 0 || a.M0 > 16 || a.N0 != 16) return false;
   if (rb != 16 && rb != 32 && rb != 64) return false;
+  if (i4 && rb == 16) return false;  // 8-byte rhs row pieces: two rows per 16-byte load
   if (probe_only) return a.M0 < 16;  // 16-row tiles only when the whole lhs is that skinny
   if (a.M * a.M0 > 16 || a.K == 0) return false;
   // Worth it only when the rhs is long enough to stream.
   if (a.N < 16) return false;
   const int64_t lhs_stride_bytes = a.lhs_stride0 * elem_bytes;
-  const int64_t rhs_stride_bytes = a.rhs_stride0 * elem_bytes;
+  const int64_t rhs_stride_bytes = i4 ? a.rhs_stride0 / 2 : a.rhs_stride0 * elem_bytes;
+  // int4: whole steps of 128 K values only, and the 16x-scaled sums must fit int32.
+  if (i4 && (((int64_t)a.K * a.K0) % 128 != 0 || (int64_t)a.K * a.K0 >= 131072)) return false;
   if ((uintptr_t)a.lhs % 16 || (a.M > 1 && lhs_stride_bytes % 16)) return false;
   if ((uintptr_t)a.rhs % 16 || rhs_stride_bytes % 16) return false;
   if ((uintptr_t)a.out % 16 || (a.M > 1 && a.out_stride0 % 4)) return false;
@@ -184,7 +300,7 @@ bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, GemvArgs* g) {
   g->log2_M0 = lm0;
   g->rb = rb;
   g->log2_rb = log2_exact(rb);
-  g->steps = (int32_t)(((int64_t)a.K * rb + 63) / 64);
+  g->steps = i4 ? (int32_t)((int64_t)a.K * a.K0 / 128) : (int32_t)(((int64_t)a.K * rb + 63) / 64);
   g->accumulate = (a.flags & IREE_UK_FLAG_MMT4D_ACCUMULATE) ? 1 : 0;
   return true;
 }
@@ -204,6 +320,16 @@ hipError_t launch_gemv(const Mmt4dArgs& a, hipStream_t stream, const char** name
   GemvArgs g;
   if (!make_args(a, false, &kind, &g)) return hipErrorInvalidValue;
   *name = "mmt4d_gemv";
+  if (kind == kI8I4) {
+    // More than 4 lhs rows: two rhs tiles per workgroup (measured on 16 rows x
+    // 65536 x 8192: 4.5 TB/s with one, 5.9 with two, 4.9 with four).
+    if ((g.M << g.log2_M0) > 4) {
+      hipLaunchKernelGGL((mmt4d_gemv_i4_kernel<2, 8, 4>), dim3((g.N + 1) / 2), dim3(256), 0, stream, g);
+    } else {
+      hipLaunchKernelGGL((mmt4d_gemv_i4_kernel<1, 8, 4>), dim3(g.N), dim3(256), 0, stream, g);
+    }
+    return hipGetLastError();
+  }
   if (kind == kI8) return launch_kind<kI8>(g, stream);
   if (kind == kF16) return launch_kind<kF16>(g, stream);
   return launch_kind<kBF16>(g, stream);
