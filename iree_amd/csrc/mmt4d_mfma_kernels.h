@@ -747,7 +747,7 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
     constexpr int B_UNITS = RHS_I4 ? BN : 0;
     constexpr int READS = RHS_I4 ? BN + 2 * AM : 2 * (AM + BN) * PARTS;
     constexpr int LEAD = MFMAS >= 16 ? 4 : (MFMAS >= 8 ? 2 : 0);   // MFMAs ahead of the barrier
-    constexpr int TAIL_FREE = MFMAS >= 8 ? MFMAS / 4 : 0;          // MFMAs after the last read
+    constexpr int TAIL_FREE = MFMAS >= 8 ? MFMAS / 4 : (RHS_I4 ? 1 : 0);  // MFMAs after the last read
     constexpr int SLOTS = MFMAS - LEAD - TAIL_FREE;                // MFMAs that carry memory work
     static_assert(SLOTS >= 1, "no room for the memory instructions");
     static_assert(!RHS_I4 || TAIL_FREE >= 1, "nowhere to widen");
@@ -928,7 +928,8 @@ struct TileChoice {
 template <bool RHS_I4>
 int choose_tile(const MfmaArgs& m, bool direct, const TileChoice** chosen) {
   static const TileChoice kTiles[] = {
-      {4, 4, 1003.f, false}, {4, 2, 905.f, true}, {2, 2, 851.f, false}, {2, 1, 607.f, true}, {1, 1, 529.f, false}};
+      {4, 4, 1003.f, false}, {4, 2, 905.f, true}, {2, 2, 851.f, false}, {2, 1, 607.f, true}, {1, 1, 529.f, false},
+      {1, 2, 600.f, true}};
   const int64_t rows = (int64_t)m.M << m.log2_M0, cols = (int64_t)m.N << m.log2_N0;
   int best = -1;
   double best_cost = 0;
@@ -936,6 +937,10 @@ int choose_tile(const MfmaArgs& m, bool direct, const TileChoice** chosen) {
     const TileChoice& t = kTiles[i];
     if (t.direct_only && !direct) continue;
     if (RHS_I4 && t.bn < 2 && t.direct_only) continue;  // the int4 direct path needs a rhs fragment per wavefront
+    if (!RHS_I4 && t.am == 1 && t.bn == 2) continue;    // 64x128 exists for the int4 rhs only (in place of 128x64)
+    // The int4 64x64 tile exists only register-staged, at less than half the
+    // rate of the direct 64x128 one on the same problem.
+    if (RHS_I4 && direct && t.am == 1 && t.bn == 1) continue;
     const int64_t br = 64 * t.am, bc = 64 * t.bn;
     const int64_t workgroups = ((rows + br - 1) / br) * ((cols + bc - 1) / bc);
     const double cost = (double)((workgroups + 255) / 256) * (double)(br * bc) / t.efficiency;
@@ -964,6 +969,10 @@ hipError_t launch_variant(const MfmaArgs& m, hipStream_t stream, const char** na
       *name = "mmt4d_mfma_128x128";
       if (direct) return launch_direct<KIND, RHS_I4, NARROW, G, 2, 2, 4>(m, stream);
       return launch_staged<KIND, RHS_I4, NARROW, G, 2, 2, 2>(m, stream);
+    case 5:
+      *name = "mmt4d_mfma_64x128";
+      if constexpr (RHS_I4) return launch_direct<KIND, RHS_I4, NARROW, G, 1, 2, 8>(m, stream);
+      [[fallthrough]];
     case 3:
       *name = "mmt4d_mfma_128x64";
       if constexpr (!RHS_I4) return launch_direct<KIND, RHS_I4, NARROW, G, 2, 1, 8>(m, stream);

@@ -124,10 +124,13 @@ def test_float_types_ragged_256(gpu_lib, flags, M0, N0, K0, K):
     run_case(gpu_lib, flags, M, N, K, M0, N0, K0, "mmt4d_mfma_256x256", accumulate=True, out_pad=16, seed=K)
 
 
-@pytest.mark.parametrize("M,N,expect", [(226, 232, "mmt4d_mfma_256x256"), (100, 119, "mmt4d_mfma_128x128"), (9, 11, "mmt4d_mfma_64x64")])
-def test_s8s4s32_ragged(gpu_lib, M, N, expect):
+@pytest.mark.parametrize("M,N,expect,expect_staged", [(226, 232, "mmt4d_mfma_256x256", "mmt4d_mfma_256x256"),
+                                                      (100, 119, "mmt4d_mfma_128x128", "mmt4d_mfma_128x128"),
+                                                      (9, 11, "mmt4d_mfma_64x128", "mmt4d_mfma_64x64")])
+def test_s8s4s32_ragged(gpu_lib, M, N, expect, expect_staged):
     run_case(gpu_lib, abi.MMT4D_TYPE_S8S4S32, M, N, 6, 16, 16, 32, expect, accumulate=True, rhs_pad=64, offsets=(16, 64, 4), seed=M)
-    run_case(gpu_lib, abi.MMT4D_TYPE_S8S4S32, M, N, 5, 16, 16, 16, expect, seed=N)   # 8-byte rhs pieces: staged kernel
+    # 8-byte rhs pieces: the register-staged kernel, which has a 64x64 tile.
+    run_case(gpu_lib, abi.MMT4D_TYPE_S8S4S32, M, N, 5, 16, 16, 16, expect_staged, seed=N)
 
 
 # The two oblong block tiles, picked for tall-and-narrow problems (few lhs rows against many rhs rows).
@@ -160,3 +163,12 @@ def test_narrow_row_pieces_fall_back_when_the_direct_kernel_cannot_run(gpu_lib):
     # K not a multiple of the chunk, or rows not 16-byte aligned: the generic kernel, still exact.
     run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, 9, 11, 33, 16, 16, 2, "mmt4d_generic", accumulate=True)
     run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, 9, 11, 32, 16, 16, 2, "mmt4d_generic", lhs_pad=4)
+
+
+# The 64x128 block tile of the int4 rhs, picked for a few dozen lhs rows against many rhs rows.
+@pytest.mark.parametrize("M0,rows,K0,K", [(16, 64, 32, 16), (16, 48, 64, 7), (8, 40, 32, 10), (4, 36, 32, 6)])
+def test_s8s4s32_64x128_tile_ragged(gpu_lib, M0, rows, K0, K):
+    n_tiles = 28600 // 16
+    run_case(gpu_lib, abi.MMT4D_TYPE_S8S4S32, rows // M0, n_tiles, K, M0, 16, K0, "mmt4d_mfma_64x128", accumulate=True,
+             rhs_pad=64, out_pad=8, offsets=(16, 64, 4), seed=rows)
+    run_case(gpu_lib, abi.MMT4D_TYPE_S8S4S32, rows // M0, n_tiles - 3, K, M0, 16, K0, "mmt4d_mfma_64x128", seed=K)
