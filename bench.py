@@ -212,6 +212,41 @@ def _also(torch, lib, abi, synth, steps, warmup):
             "frac_of_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
     del rhs_set
 
+    # The same with int4 weights (s8s4s32, tiles M0 x 16 x 32): N = 28672,
+    # K = 8192, 117 MB of nibbles per rhs copy, three copies rotated. The
+    # checksum of the M0 = 16 result is compared with torch's on the widened
+    # weights.
+    n_i4, k_i4 = 28672, 8192
+    rhs_i4 = [torch.from_numpy(synth.uniform_int4_packed(12, i, n_i4 * k_i4).view(np.int8)).cuda() for i in range(3)]
+    for m0 in (1, 16):
+        lhs = torch.from_numpy(synth.uniform_int8(12, 10 + m0, m0 * k_i4)).cuda()
+        outs = torch.zeros((n_i4 // 16) * m0 * 16, dtype=torch.int32, device="cuda")
+        ps = [_mmt4d_params(abi, lhs.data_ptr(), r.data_ptr(), outs.data_ptr(), 1, n_i4 // 16, k_i4 // 32, m0, 16, 32,
+                            abi.MMT4D_TYPE_S8S4S32) for r in rhs_i4]
+        state = {"i": 0}
+
+        def step_i4():
+            lib.iree_uk_mmt4d_p(C.byref(ps[state["i"] % 3]))
+            state["i"] += 1
+        ms, _ = _time_launches(torch, step_i4, max(steps, 6), warmup)
+        nbytes = n_i4 * k_i4 // 2 + m0 * k_i4 + n_i4 * m0 * 4
+        entry = {"kernel": lib.iree_uk_mi355x_last_kernel().decode(), "ms": round(ms, 5),
+                 "value": round(nbytes / ms / 1e6, 1), "unit": "GB/s",
+                 "frac_of_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+        if m0 == 16:
+            lib.iree_uk_mmt4d_p(C.byref(ps[0]))
+            torch.cuda.synchronize()
+            r = rhs_i4[0].to(torch.int16)
+            w = torch.stack([r & 0xF, (r >> 4) & 0xF], dim=1).reshape(-1)
+            w = ((w ^ 8) - 8).to(torch.float64).view(n_i4 // 16, k_i4 // 32, 16, 32)
+            a = lhs.view(k_i4 // 32, 16, 32).to(torch.float64)
+            # sum over all outputs = sum_k (column sums of a) * (column sums of w), exact in float64
+            want = (a.sum(dim=1) * w.sum(dim=(0, 2))).sum().item()
+            entry["checksum_verified"] = bool(outs.to(torch.float64).sum().item() == want)
+            del r, w, a
+        res["mmt4d_s8s4s32_skinny_M%d_N28672_K8192" % m0] = entry
+    del rhs_i4
+
     # pack / unpack f32 [8191, 8190] <-> [512, 8190, 16, 1]; two buffer sets rotated
     # (each set is 537 MB, beyond the last-level cache).
     R, Cc = 8191, 8190
