@@ -9,10 +9,10 @@
 // in LDS:
 //   pack:    2-D rows -> LDS (row-major, padded pitch) -> tiled runs (128-bit)
 //   unpack:  tiled runs (128-bit) -> LDS -> 2-D rows
-// The 2-D side uses the widest vector (16, 8 or 4 bytes, else one element)
-// that the row alignment allows. Element values are never interpreted: the
-// kernels move bytes, so results are bit-exact by construction; padding is the
-// low bytes of padding_value (pack.h:15-24).
+// The 2-D side uses 16-byte vectors whatever the alignment of the rows.
+// Element values are never interpreted: the kernels move bytes, so results are
+// bit-exact by construction; padding is the low bytes of padding_value
+// (pack.h:15-24).
 //
 // With an inner transpose the tiled side's 16 contiguous bytes are 16 / E
 // consecutive ROWS of one column. For 4-byte elements that is four 32-bit LDS
@@ -122,9 +122,9 @@ __device__ __forceinline__ void block_of(const TiledArgs& a, int32_t linear, int
   *block1 = i / rows_here;
 }
 
-// 16 bytes that only need 4-byte alignment: the hardware's multi-dword global
-// accesses do not require more, the C++ type system would.
-struct __attribute__((packed, aligned(4))) Dwords4 {
+// 16 bytes without an alignment requirement: the hardware's multi-dword
+// global accesses have none, the C++ type system would.
+struct __attribute__((packed, aligned(1))) Dwords4 {
   uint32_t x, y, z, w;
 };
 
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
           // Every byte is read once: streaming (non-temporal) accesses on both
           // sides leave the caches to the other side's partial lines.
           if constexpr (W == 16) {
-            typedef int v4a4 __attribute__((ext_vector_type(4), aligned(4)));
+            typedef int v4a4 __attribute__((ext_vector_type(4), aligned(1)));
             const v4a4 t = __builtin_nontemporal_load((const v4a4*)g);
             regs[u].vec = Dwords4{(uint32_t)t.x, (uint32_t)t.y, (uint32_t)t.z, (uint32_t)t.w};
           } else {
@@ -235,8 +235,8 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
         if (row < a.size0 && col + EPV <= a.size1) {
           // Whole vectors inside the matrix: written once, not read here.
           if constexpr (W == 16) {
-            typedef int v4 __attribute__((ext_vector_type(4)));
-            __builtin_nontemporal_store(v4{(int)regs[u].vec.x, (int)regs[u].vec.y, (int)regs[u].vec.z, (int)regs[u].vec.w}, (v4*)g);
+            typedef int v4a1 __attribute__((ext_vector_type(4), aligned(1)));
+            __builtin_nontemporal_store(v4a1{(int)regs[u].vec.x, (int)regs[u].vec.y, (int)regs[u].vec.z, (int)regs[u].vec.w}, (v4a1*)g);
           } else if constexpr (W == 8) {
             typedef int v2 __attribute__((ext_vector_type(2)));
             __builtin_nontemporal_store(v2{(int)regs[u].vec.x, (int)regs[u].vec.y}, (v2*)g);
@@ -381,7 +381,7 @@ __global__ __launch_bounds__(256) void pack_transposing_wide_kernel(const TiledA
       const int64_t row = row_base + patch_row[u] + lane_row * RQ + j, col = col_base + patch_col[u] + cg * VE;
       const uint8_t* g = a.src + (row * a.flat_stride0 + col) * E;
       if (row < a.size0 && col + VE <= a.size1) {
-        typedef int v4a4 __attribute__((ext_vector_type(4), aligned(4)));
+        typedef int v4a4 __attribute__((ext_vector_type(4), aligned(1)));
         const v4a4 t = __builtin_nontemporal_load((const v4a4*)g);
         regs[u][j].dword[0] = t.x; regs[u][j].dword[1] = t.y; regs[u][j].dword[2] = t.z; regs[u][j].dword[3] = t.w;
       } else {
@@ -481,7 +481,7 @@ __global__ __launch_bounds__(256) void pack_transposing_kernel(const TiledArgs a
       const int64_t row = row_base + row0[u] + j, col = col_base + col0[u];
       const uint8_t* g = a.src + (row * a.flat_stride0 + col) * E;
       if (row < a.size0 && col + VE <= a.size1) {
-        typedef int v4a4 __attribute__((ext_vector_type(4), aligned(4)));
+        typedef int v4a4 __attribute__((ext_vector_type(4), aligned(1)));
         const v4a4 t = __builtin_nontemporal_load((const v4a4*)g);
         regs[u][j].dword[0] = t.x; regs[u][j].dword[1] = t.y; regs[u][j].dword[2] = t.z; regs[u][j].dword[3] = t.w;
       } else {
@@ -656,26 +656,20 @@ bool make_plan(const uint8_t* flat, const uint8_t* tiled, int64_t flat_stride0, 
   a.log2_br = log2_exact(br);
   a.log2_bc = log2_exact(bc);
 
-  // Vector width on the 2-D side from the alignment shared by all rows:
-  // 16-byte vectors need 4-byte alignment only.
-  int w = largest_pow2_dividing((uintptr_t)flat, 4);
-  if (size0 > 1) {
-    const int ws = largest_pow2_dividing((uint64_t)(flat_stride0 * E), 4);
-    w = ws < w ? ws : w;
-  }
-  if (w < E) return false;
-  // Loads may be under-aligned 16-byte vectors; stores are faster when aligned,
-  // so unpack uses the widest vector that the rows are aligned to.
-  if (!for_unpack) {
-    plan->flat_vec_bytes = w == 4 ? 16 : w;
-  } else {
-    int wa = largest_pow2_dividing((uintptr_t)flat, 16);
+  // 2-D side: 16-byte vectors whatever the alignment of the rows (global memory
+  // accesses need none; for loads this is worth up to 1.6x on rows that are
+  // only byte aligned, for stores 4-9 % over the widest aligned vector).
+  // Elements themselves must be aligned: edges are handled element by element.
+  {
+    int w = largest_pow2_dividing((uintptr_t)flat, 4);
     if (size0 > 1) {
-      const int ws = largest_pow2_dividing((uint64_t)(flat_stride0 * E), 16);
-      wa = ws < wa ? ws : wa;
+      const int ws = largest_pow2_dividing((uint64_t)(flat_stride0 * E), 4);
+      w = ws < w ? ws : w;
     }
-    plan->flat_vec_bytes = wa;
+    if (w < E) return false;
   }
+  (void)for_unpack;
+  plan->flat_vec_bytes = 16;
 
   // Contiguous LDS piece on the tiled side.
   int piece = tr_inner ? E : (int)((T1 * E) < 16 ? (T1 * E) : 16);
@@ -849,14 +843,8 @@ hipError_t launch_pw(const Plan& p, hipStream_t stream) {
 
 template <int E, bool UNPACK>
 hipError_t launch_e(const Plan& p, hipStream_t stream) {
-  switch (p.flat_vec_bytes) {
-    case 16: return launch_pw<E, 16, UNPACK>(p, stream);
-    case 8: return launch_pw<E, 8, UNPACK>(p, stream);
-    case 4: return launch_pw<E, 4, UNPACK>(p, stream);
-    case 2: if constexpr (E <= 2) return launch_pw<E, 2, UNPACK>(p, stream); return hipErrorInvalidValue;
-    case 1: if constexpr (E == 1) return launch_pw<E, 1, UNPACK>(p, stream); return hipErrorInvalidValue;
-    default: return hipErrorInvalidValue;
-  }
+  if (p.flat_vec_bytes != 16) return hipErrorInvalidValue;
+  return launch_pw<E, 16, UNPACK>(p, stream);
 }
 
 template <bool UNPACK>

@@ -352,7 +352,7 @@ def test_pack_nonzero_padding_value_and_i8_operand_layouts(gpu_lib, oracle_lib):
         q = _pack_params(d_src.data_ptr(), d_out.data_ptr(), R, Cc, o0, o1, t0, t1, flags, pad=0x115A)
         q.flags = abi.PACK_TYPE_I8I8 | flags
         gpu_lib.iree_uk_pack_p(C.byref(q))
-        assert gpu_lib.iree_uk_mi355x_last_kernel() == b"pack_tiled"
+        assert gpu_lib.iree_uk_mi355x_last_kernel() == (b"pack_transposing" if flags else b"pack_tiled")
         assert np.array_equal(d_out.cpu().numpy(), want)
 
 

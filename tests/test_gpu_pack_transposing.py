@@ -73,8 +73,8 @@ def test_pack_inner_transpose_small_elements(gpu_lib, oracle_lib, case):
         raise AssertionError("%d bytes differ, first at %d: got %d want %d" % (bad.size, bad[0], got[bad[0]], want[bad[0]]))
 
 
-def test_pack_inner_transpose_rows_not_dword_aligned_use_the_older_kernel(gpu_lib, oracle_lib):
-    # Row stride 1001 bytes: rows are only byte aligned, no 16-byte loads.
+def test_pack_inner_transpose_rows_only_byte_aligned(gpu_lib, oracle_lib):
+    # Row stride 1001 bytes: rows are only byte aligned; the 16-byte loads do not mind.
     rows, cols, t0, t1 = 300, 1001, 16, 16
     flags = abi.PACK_TYPE_I8I8 | TI | TO
     o0, o1 = -(-rows // t0), -(-cols // t1)
@@ -95,5 +95,5 @@ def test_pack_inner_transpose_rows_not_dword_aligned_use_the_older_kernel(gpu_li
     d_src = torch.from_numpy(src).cuda()
     d_out = torch.full((want.size,), 0x11, dtype=torch.int8, device="cuda")
     gpu_lib.iree_uk_pack_p(C.byref(params(d_src.data_ptr(), d_out.data_ptr())))
-    assert gpu_lib.iree_uk_mi355x_last_kernel() == b"pack_tiled"
+    assert gpu_lib.iree_uk_mi355x_last_kernel() == b"pack_transposing"
     assert np.array_equal(d_out.cpu().numpy(), want)
