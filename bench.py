@@ -146,27 +146,34 @@ def _also(torch, lib, abi, synth, steps, warmup):
     mm("mmt4d_s8s8s32_4096_8x8x4_all_zero_operands_clock_check", abi.MMT4D_TYPE_S8S8S32, 512, 512, 1024, 8, 8, 4,
        zl, zl, torch.int32, PEAK_INT8_TOPS, "TOP/s")
     del zl
-    # What the int8 matrix pipe sustains on this device, measured by the
+    # What the matrix pipe sustains on this device, measured by the
     # library's probe: the 256x256 kernel's inner-loop instruction mix with no
-    # HBM traffic, no prologue and no epilogue, on all-zero and on the headline's
-    # uniformly random operand bytes, without and with the loop's LDS reads,
-    # loads to LDS and barrier. A ceiling to read the headline against, not a
-    # result: the cycle count per step is the same in all four, the clock is not.
+    # HBM traffic, no prologue and no epilogue, on all-zero bytes, on the
+    # headline's uniformly random int8 and on the f16 / bf16 configurations'
+    # operands, without and with the loop's LDS reads, loads to LDS and barrier.
+    # A ceiling to read the mmt4d figures against, not a result: the cycle count
+    # per step is the same in all of them, the clock is not.
     probe = {}
     rnd = torch.from_numpy(synth.uniform_int8(0, 0, 2 << 20)).cuda()
     zer = torch.zeros(2 << 20, dtype=torch.int8, device="cuda")
-    for data_name, buf in (("zero_bytes", zer), ("random_bytes", rnd)):
+    f16 = f16_operand(3, 0, 1 << 20, 1.0 / 64)              # the f16 configuration's operand distribution
+    bf16 = f16_operand(4, 10, 1 << 20, 0.02, bf16=True)     # the bf16 configuration's weights
+    for type_flag, peak, unit, data_name, buf in (
+            (abi.MMT4D_TYPE_S8S8S32, PEAK_INT8_TOPS, "TOP/s", "int8_zero_bytes", zer),
+            (abi.MMT4D_TYPE_S8S8S32, PEAK_INT8_TOPS, "TOP/s", "int8_uniform_random", rnd),
+            (abi.MMT4D_TYPE_F16F16F32, PEAK_F16_TFLOPS, "TFLOP/s", "f16_normal_over_64", f16),
+            (abi.MMT4D_TYPE_BF16BF16F32, PEAK_F16_TFLOPS, "TFLOP/s", "bf16_normal_sigma_0.02", bf16)):
         for traffic in (0, 1):
             tops, mhz = C.c_double(), C.c_double()
-            rc = lib.iree_uk_mi355x_probe_int8_matrix_pipe(buf.data_ptr(), buf.numel(), traffic, 4096,
-                                                           C.byref(tops), C.byref(mhz))
+            rc = lib.iree_uk_mi355x_probe_matrix_pipe(type_flag, buf.data_ptr(), buf.numel() * buf.element_size(),
+                                                      traffic, 4096, C.byref(tops), C.byref(mhz))
             if rc != 0:
                 raise RuntimeError("matrix pipe probe failed: HIP error %d" % rc)
             probe["%s_%s" % (data_name, "with_lds_traffic" if traffic else "mfma_only")] = {
-                "value": round(tops.value, 1), "unit": "TOP/s", "frac_of_peak": round(tops.value / PEAK_INT8_TOPS, 4),
+                "value": round(tops.value, 1), "unit": unit, "frac_of_peak": round(tops.value / peak, 4),
                 "shader_mhz": round(mhz.value)}
-    res["int8_matrix_pipe_sustained_rate_probe"] = probe
-    del rnd, zer
+    res["matrix_pipe_sustained_rate_probe"] = probe
+    del rnd, zer, f16, bf16
     # f32f32f32 4096^3 with the tile shape query_tile_sizes hands out for f32 (16x16x4).
     mm("mmt4d_f32f32f32_4096_16x16x4", abi.MMT4D_TYPE_F32F32F32, 256, 256, 1024, 16, 16, 4,
        torch.from_numpy(synth.normal_f32(6, 0, n, 1.0)).cuda(), torch.from_numpy(synth.normal_f32(6, 1, n, 1.0)).cuda(),

@@ -1,10 +1,12 @@
-// A measuring stick, not part of the matmul path: what the int8 matrix pipe of
-// the device sustains on given operand bytes. One workgroup of four wavefronts
-// per compute unit runs the inner loop of the 256x256 mmt4d kernel stripped to
-// its instruction mix: per step 32 independent 32x32x32 int8 MFMAs per
-// wavefront (a 4x4 grid of accumulator fragments, two K-steps), optionally
-// with the step's memory instructions (16 128-bit LDS reads that feed the next
-// step's operands, 8 loads of 1 KiB straight to LDS, one workgroup barrier).
+// A measuring stick, not part of the matmul path: what the matrix pipe of the
+// device sustains on given operand bytes, for int8, f16 or bf16 operands. One
+// workgroup of four wavefronts per compute unit runs the inner loop of the
+// 256x256 mmt4d kernel stripped to its instruction mix: per step 32
+// independent MFMAs per wavefront (32x32x32 int8 or 32x32x16 f16/bf16: a 4x4
+// grid of accumulator fragments, two K-steps of 16 operand bytes per lane),
+// optionally with the step's memory instructions (16 128-bit LDS reads that
+// feed the next step's operands, 8 loads of 1 KiB straight to LDS, one
+// workgroup barrier).
 // There is no HBM traffic to speak of (the loads hit in cache) and no
 // prologue or epilogue, so the rate it reports is a ceiling for any kernel
 // built on these instructions.
@@ -22,18 +24,40 @@ namespace {
 
 typedef int v4i32 __attribute__((ext_vector_type(4)));
 typedef int v16i32 __attribute__((ext_vector_type(16)));
+typedef float v16f32 __attribute__((ext_vector_type(16)));
+typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
+typedef __bf16 v8bf16 __attribute__((ext_vector_type(8)));
+
+enum ProbeKind { kProbeI8 = 0, kProbeF16 = 1, kProbeBF16 = 2 };
+template <int KIND> struct ProbeAcc { typedef v16i32 type; };
+template <> struct ProbeAcc<kProbeF16> { typedef v16f32 type; };
+template <> struct ProbeAcc<kProbeBF16> { typedef v16f32 type; };
+
+template <int KIND>
+__device__ __forceinline__ typename ProbeAcc<KIND>::type probe_mfma(uint4 a, uint4 b, typename ProbeAcc<KIND>::type c) {
+  if constexpr (KIND == kProbeI8) {
+    return __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(v4i32, a), __builtin_bit_cast(v4i32, b), c, 0, 0, 0);
+  } else if constexpr (KIND == kProbeF16) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8f16, a), __builtin_bit_cast(v8f16, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf16, a), __builtin_bit_cast(v8bf16, b), c, 0, 0, 0);
+  }
+}
+
+__device__ __forceinline__ int32_t accumulator_bits(int32_t v) { return v; }
+__device__ __forceinline__ int32_t accumulator_bits(float v) { return __float_as_int(v); }
 
 extern __shared__ uint4 probe_lds[];
 
 constexpr int kLdsBytes = 128 * 1024;      // lower half: what the LDS reads fetch; upper half: where the loads land
 constexpr int kOperandBytesNeeded = 2 << 20;
 
-template <bool TRAFFIC>
+template <int KIND, bool TRAFFIC>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void probe_kernel(const uint8_t* src, int32_t* sink, int steps, long long* cycles) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  v16i32 acc[4][4];
+  typename ProbeAcc<KIND>::type acc[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -77,8 +101,7 @@ void probe_kernel(const uint8_t* src, int32_t* sink, int steps, long long* cycle
 #pragma unroll
         for (int u = slot * 16 / 24; u < (slot + 1) * 16 / 24; ++u) n[u] = *(const uint4*)(read_base + u * 1024);
       }
-      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(v4i32, c[8 * kk + 4 + j]),
-                                                        __builtin_bit_cast(v4i32, c[8 * kk + i]), acc[i][j], 0, 0, 0);
+      acc[i][j] = probe_mfma<KIND>(c[8 * kk + 4 + j], c[8 * kk + i], acc[i][j]);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -94,18 +117,37 @@ void probe_kernel(const uint8_t* src, int32_t* sink, int steps, long long* cycle
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) x ^= acc[i][j][v];
-  // Keeps the accumulators alive; practically never true.
-  if (x == 0x7654321 && steps < 0) sink[0] = x;
+      for (int v = 0; v < 16; ++v) x ^= accumulator_bits(acc[i][j][v]);
+  // Keeps the accumulators alive: practically never true, but not provably so.
+  if (x == 0x7654321) sink[0] = x;
   if (threadIdx.x == 0 && blockIdx.x == 0) cycles[0] = t1 - t0;
 }
 
 }  // namespace
 
-UK_API int iree_uk_mi355x_probe_int8_matrix_pipe(const void* operand_bytes, long long operand_size, int memory_traffic,
-                                                 int steps, double* tera_ops_per_second, double* shader_mhz) {
+UK_API int iree_uk_mi355x_probe_matrix_pipe(uint32_t mmt4d_type, const void* operand_bytes, long long operand_size,
+                                            int memory_traffic, int steps, double* tera_ops_per_second,
+                                            double* shader_mhz) {
   if (operand_bytes == nullptr || operand_size < kOperandBytesNeeded || steps < 2 || (steps & 1)) {
     return (int)hipErrorInvalidValue;
+  }
+  void (*kernel)(const uint8_t*, int32_t*, int, long long*) = nullptr;
+  double ops_per_mfma = 0;
+  switch (mmt4d_type) {
+    case 0x02:  // IREE_UK_FLAG_MMT4D_TYPE_S8S8S32
+      kernel = memory_traffic ? probe_kernel<kProbeI8, true> : probe_kernel<kProbeI8, false>;
+      ops_per_mfma = 2.0 * 32 * 32 * 32;
+      break;
+    case 0x03:  // IREE_UK_FLAG_MMT4D_TYPE_F16F16F32
+      kernel = memory_traffic ? probe_kernel<kProbeF16, true> : probe_kernel<kProbeF16, false>;
+      ops_per_mfma = 2.0 * 32 * 32 * 16;
+      break;
+    case 0x05:  // IREE_UK_FLAG_MMT4D_TYPE_BF16BF16F32
+      kernel = memory_traffic ? probe_kernel<kProbeBF16, true> : probe_kernel<kProbeBF16, false>;
+      ops_per_mfma = 2.0 * 32 * 32 * 16;
+      break;
+    default:
+      return (int)hipErrorInvalidValue;
   }
   int device = 0, cus = 0;
   hipError_t e = hipGetDevice(&device);
@@ -117,7 +159,6 @@ UK_API int iree_uk_mi355x_probe_int8_matrix_pipe(const void* operand_bytes, long
   hipEvent_t begin = nullptr, end = nullptr;
   float ms = 0.f;
   long long cycles = 0;
-  auto kernel = memory_traffic ? probe_kernel<true> : probe_kernel<false>;
   e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
   if (e == hipSuccess) e = hipEventCreate(&begin);
   if (e == hipSuccess) e = hipEventCreate(&end);
@@ -138,7 +179,7 @@ UK_API int iree_uk_mi355x_probe_int8_matrix_pipe(const void* operand_bytes, long
   if (end) (void)hipEventDestroy(end);
   (void)hipFree(scratch);
   if (e != hipSuccess) return (int)e;
-  const double ops = (double)cus * 4 * steps * 32 * (2.0 * 32 * 32 * 32);
+  const double ops = (double)cus * 4 * steps * 32 * ops_per_mfma;
   if (tera_ops_per_second) *tera_ops_per_second = ops / (ms * 1e-3) / 1e12;
   if (shader_mhz) *shader_mhz = (double)cycles / (ms * 1e3);
   return 0;

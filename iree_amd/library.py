@@ -51,9 +51,9 @@ def load():
     l.iree_uk_mi355x_version.restype = C.c_int
     l.iree_uk_mi355x_multi_mma_i32_16x16x64_i8.argtypes = [vp, vp, vp, C.c_longlong, C.c_longlong] + [C.c_int32] * 6
     l.iree_uk_mi355x_multi_mma_i32_16x16x64_i8.restype = C.c_int
-    l.iree_uk_mi355x_probe_int8_matrix_pipe.argtypes = [vp, C.c_longlong, C.c_int, C.c_int,
-                                                        C.POINTER(C.c_double), C.POINTER(C.c_double)]
-    l.iree_uk_mi355x_probe_int8_matrix_pipe.restype = C.c_int
+    l.iree_uk_mi355x_probe_matrix_pipe.argtypes = [C.c_uint32, vp, C.c_longlong, C.c_int, C.c_int,
+                                                   C.POINTER(C.c_double), C.POINTER(C.c_double)]
+    l.iree_uk_mi355x_probe_matrix_pipe.restype = C.c_int
     l.iree_uk_mi355x_init.argtypes = [C.c_int]
     l.iree_uk_mi355x_init.restype = C.c_int
     l.iree_uk_mi355x_set_stream.argtypes = [vp, C.c_int]
