@@ -448,13 +448,18 @@ __global__ __launch_bounds__(256) void pack_transposing_wide_kernel(const TiledA
 }
 
 // Pack with an inner transpose for 1- and 2-byte elements (see the top of the
-// file). Needs rows that are 4-byte aligned and tiles at least 4 / E rows tall.
-template <int E>
+// file). A dword of the tiled side is RQ consecutive rows of 4 / (E * RQ)
+// adjacent columns: RQ = 4 / E rows of one column for tiles at least that
+// tall, or, for int8 tiles two rows tall (the [N0][2] layouts of the x86
+// dot-product tiles), 2 rows of 2 columns.
+template <int E, int RQ>
 __global__ __launch_bounds__(256) void pack_transposing_kernel(const TiledArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   typedef typename std::conditional<E == 1, uint8_t, uint16_t>::type elem_t;
-  constexpr int RQ = 4 / E;   // rows whose elements of one column make up a dword
-  constexpr int VE = 16 / E;  // columns per 16-byte vector
+  static_assert((E == 1 && (RQ == 4 || RQ == 2)) || (E == 2 && RQ == 2), "rows per dword");
+  constexpr int CQ = 4 / (E * RQ);  // columns per dword
+  constexpr int NOUT = 4 / E / CQ;  // dwords made from one dword of each of the RQ rows
+  constexpr int VE = 16 / E;        // columns per 16-byte vector
   constexpr int UNITS = kBlockBytes / (RQ * 16) / 256;
   constexpr int TILED_PER_THREAD = kBlockBytes / 16 / 256;
 
@@ -498,8 +503,8 @@ __global__ __launch_bounds__(256) void pack_transposing_kernel(const TiledArgs a
   for (int u = 0; u < UNITS; ++u) {
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-      uint32_t out[RQ];
-      if constexpr (E == 1) {
+      uint32_t out[NOUT];
+      if constexpr (E == 1 && RQ == 4) {
         const uint32_t ra = regs[u][0].dword[k], rb = regs[u][1].dword[k], rc = regs[u][2].dword[k], rd = regs[u][3].dword[k];
         const uint32_t ab_lo = __builtin_amdgcn_perm(rb, ra, 0x05010400u), ab_hi = __builtin_amdgcn_perm(rb, ra, 0x07030602u);
         const uint32_t cd_lo = __builtin_amdgcn_perm(rd, rc, 0x05010400u), cd_hi = __builtin_amdgcn_perm(rd, rc, 0x07030602u);
@@ -507,14 +512,19 @@ __global__ __launch_bounds__(256) void pack_transposing_kernel(const TiledArgs a
         out[1] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x07060302u);
         out[2] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x05040100u);
         out[3] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x07060302u);
+      } else if constexpr (E == 1) {
+        // Two rows: bytes (column c, row 0), (c, 1), (c + 1, 0), (c + 1, 1).
+        const uint32_t ra = regs[u][0].dword[k], rb = regs[u][1].dword[k];
+        out[0] = __builtin_amdgcn_perm(rb, ra, 0x05010400u);
+        out[1] = __builtin_amdgcn_perm(rb, ra, 0x07030602u);
       } else {
         const uint32_t ra = regs[u][0].dword[k], rb = regs[u][1].dword[k];
         out[0] = __builtin_amdgcn_perm(rb, ra, 0x05040100u);
         out[1] = __builtin_amdgcn_perm(rb, ra, 0x07060302u);
       }
 #pragma unroll
-      for (int i = 0; i < RQ; ++i) {
-        const int32_t e = tiled_index_tr_inner(a, row0[u], col0[u] + RQ * k + i);
+      for (int i = 0; i < NOUT; ++i) {
+        const int32_t e = tiled_index_tr_inner(a, row0[u], col0[u] + (4 / E) * k + CQ * i);
         *(uint32_t*)(lds + skewed(a, (uint32_t)e * E)) = out[i];
       }
     }
@@ -702,11 +712,12 @@ struct TransposingChoice {
   int32_t log2_lpr, log2_period, pad_bytes;
 };
 
-void choose_transposing(TiledArgs* a, int elem_bytes) {
+void choose_transposing(TiledArgs* a, int elem_bytes, int rq) {
   static std::mutex mutex;
   static std::vector<TransposingChoice> known;
   const uint32_t key = (uint32_t)elem_bytes | (uint32_t)a->log2_t0 << 4 | (uint32_t)a->log2_t1 << 8 |
-                       (uint32_t)a->log2_br << 12 | (uint32_t)a->log2_bc << 17 | (uint32_t)a->tr_outer << 22;
+                       (uint32_t)a->log2_br << 12 | (uint32_t)a->log2_bc << 17 | (uint32_t)a->tr_outer << 22 |
+                       (uint32_t)rq << 23;
   std::lock_guard<std::mutex> lock(mutex);
   for (const TransposingChoice& c : known) {
     if (c.key == key) {
@@ -714,7 +725,8 @@ void choose_transposing(TiledArgs* a, int elem_bytes) {
       return;
     }
   }
-  const int rq = 4 / elem_bytes, ve = 16 / elem_bytes;
+  const int ve = 16 / elem_bytes;
+  const int cq = 4 / (elem_bytes * rq);
   const int log2_cg = a->log2_bc + (elem_bytes == 2 ? 1 : 0) - 4;
   TransposingChoice best{key, 0, 14, 0};
   long best_cost = -1;
@@ -724,7 +736,7 @@ void choose_transposing(TiledArgs* a, int elem_bytes) {
       for (t.pad_bytes = 0; t.pad_bytes <= 64; t.pad_bytes += 16) {
         if (t.log2_period == 14 && t.pad_bytes) break;  // one period: padding changes nothing
         long cost = 0;
-        for (int i = 0; i < ve; ++i) {
+        for (int i = 0; i < ve; i += cq) {
           for (int half = 0; half < 2; ++half) {
             int hits[32] = {0};
             int worst = 0;
@@ -799,20 +811,27 @@ void choose_transposing_wide(TiledArgs* a, int elem_bytes) {
 }
 
 // Whether one of the transposing kernels takes the planned call (0: no,
-// 1: pack_transposing_kernel, 2: pack_transposing_wide_kernel); sets it up.
+// 1: pack_transposing_kernel, 2: pack_transposing_wide_kernel, 3:
+// pack_transposing_kernel for int8 tiles two rows tall); sets it up.
 int plan_transposing(Plan* p) {
   TiledArgs& a = p->args;
   const int E = p->elem_bytes;
   if (!a.tr_inner || E > 2 || p->flat_vec_bytes != 16) return 0;
   const int log2_e = E == 2 ? 1 : 0;
   const int log2_rq = 2 - log2_e, log2_ve = 4 - log2_e;
-  if (a.log2_t0 < log2_rq || a.log2_bc + log2_e < 4) return 0;
+  if (a.log2_bc + log2_e < 4) return 0;
+  if (E == 1 && a.log2_t0 == 1 && a.log2_t1 >= 1 && a.log2_br >= 1) {
+    choose_transposing(&a, E, 2);
+    p->lds_bytes = skewed(a, kBlockBytes - 16) + 16;
+    return 3;
+  }
+  if (a.log2_t0 < log2_rq) return 0;
   int which = 1;
   if (a.log2_t0 >= log2_ve && a.log2_bc + log2_e >= 8 && a.log2_br >= log2_ve) {
     which = 2;
     choose_transposing_wide(&a, E);
   } else {
-    choose_transposing(&a, E);
+    choose_transposing(&a, E, 4 / E);
   }
   p->lds_bytes = skewed(a, kBlockBytes - 16) + 16;
   return which;
@@ -877,10 +896,12 @@ hipError_t launch_pack(const PackArgs& a, hipStream_t stream, const char** name)
       hipLaunchKernelGGL(pack_transposing_wide_kernel<1>, grid, block, plan.lds_bytes, stream, plan.args);
     } else if (which == 2) {
       hipLaunchKernelGGL(pack_transposing_wide_kernel<2>, grid, block, plan.lds_bytes, stream, plan.args);
+    } else if (which == 3) {
+      hipLaunchKernelGGL((pack_transposing_kernel<1, 2>), grid, block, plan.lds_bytes, stream, plan.args);
     } else if (plan.elem_bytes == 1) {
-      hipLaunchKernelGGL(pack_transposing_kernel<1>, grid, block, plan.lds_bytes, stream, plan.args);
+      hipLaunchKernelGGL((pack_transposing_kernel<1, 4>), grid, block, plan.lds_bytes, stream, plan.args);
     } else {
-      hipLaunchKernelGGL(pack_transposing_kernel<2>, grid, block, plan.lds_bytes, stream, plan.args);
+      hipLaunchKernelGGL((pack_transposing_kernel<2, 2>), grid, block, plan.lds_bytes, stream, plan.args);
     }
     return hipGetLastError();
   }

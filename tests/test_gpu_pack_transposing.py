@@ -23,7 +23,9 @@ CASES = [
     (abi.PACK_TYPE_I8I8, 1021, 3001 + 3, 64, 16, TI | TO, 0, 0),     # rhs of 16x16x64: [n][k][16][64]
     (abi.PACK_TYPE_I8I8, 1021, 3004, 4, 8, TI | TO, 0, 0),           # rhs of 8x8x4: tiles narrower than a vector
     (abi.PACK_TYPE_I8I8, 777, 1000, 32, 16, TI, 24, 0),              # no outer transpose, row stride with a gap
-    (abi.PACK_TYPE_I8I8, 513, 2052, 2, 16, TI | TO, 0, 0),           # tile shorter than 4 rows: the older kernel
+    (abi.PACK_TYPE_I8I8, 513, 2052, 2, 16, TI | TO, 0, 0),           # [16][2] tiles (x86 dot-product rhs): 2 rows x 2 columns per dword
+    (abi.PACK_TYPE_I8I8, 1001, 777, 2, 8, TI, 5, 16),                # [8][2] tiles, odd row stride
+    (abi.PACK_TYPE_I8I8, 300, 500, 1, 16, TI | TO, 0, 0),            # one-row int8 tiles: the older kernel
     (abi.PACK_TYPE_I8I8, 300, 4100, 64, 64, TI | TO, 0, 64),         # 4 KiB tiles (the reference's limit), outer stride with a gap
     (abi.PACK_TYPE_I8I8, 2050, 260, 16, 2, TI, 0, 0),                # 2-column tiles
     (abi.PACK_TYPE_F16F16, 1000, 2002, 16, 16, TI | TO, 0, 0),
@@ -65,7 +67,7 @@ def test_pack_inner_transpose_small_elements(gpu_lib, oracle_lib, case):
     d_src = torch.from_numpy(src).cuda()
     d_out = torch.full((n_out * e,), 0x77, dtype=torch.int8, device="cuda")
     gpu_lib.iree_uk_pack_p(C.byref(params(d_src.data_ptr(), d_out.data_ptr())))
-    expected_kernel = b"pack_transposing" if t0 * e >= 4 else b"pack_tiled"
+    expected_kernel = b"pack_transposing" if t0 * e >= 4 or (e == 1 and t0 == 2) else b"pack_tiled"
     assert gpu_lib.iree_uk_mi355x_last_kernel() == expected_kernel
     got = d_out.cpu().numpy()
     if not np.array_equal(got, want):
