@@ -878,14 +878,35 @@ hipError_t launch_plan(const Plan& p, hipStream_t stream) {
 
 }  // namespace
 
-hipError_t launch_pack(const PackArgs& a, hipStream_t stream, const char** name) {
+hipError_t launch_pack(const PackArgs& original, hipStream_t stream, const char** name) {
   Plan plan;
-  const bool tr_inner = a.flags & IREE_UK_FLAG_PACK_TRANSPOSE_INNER;
+  PackArgs a = original;
+  bool tr_inner = a.flags & IREE_UK_FLAG_PACK_TRANSPOSE_INNER;
   const bool tr_outer = a.flags & IREE_UK_FLAG_PACK_TRANSPOSE_OUTER;
+  // Tiles one column wide are consecutive rows of that column whichever way the
+  // inner dimensions are ordered; and int8 tiles two columns wide are tiles one
+  // column wide of 2-byte elements when everything else is even. Both are put
+  // in the inner-transposed form, which for 1- and 2-byte elements has the
+  // register-transposing kernels (int8 [M1][K1][16][2] lhs layouts: 4.8 ->
+  // 5.5 TB/s).
+  if (!tr_inner && a.elem_bytes == 1 && a.out_size3 == 2 && a.in_stride1 == 1 && a.in_size1 % 2 == 0 &&
+      a.in_stride0 % 2 == 0 && a.out_stride0 % 2 == 0 && (uintptr_t)a.in % 2 == 0) {
+    a.elem_bytes = 2;
+    a.in_size1 /= 2;
+    a.in_stride0 /= 2;
+    a.out_stride0 /= 2;
+    a.out_size3 = 1;
+    a.padding_value = (a.padding_value & 0xFF) * 0x0101u;
+  }
+  if (!tr_inner && a.out_size3 == 1 && a.elem_bytes <= 2) {
+    a.out_size3 = a.out_size2;
+    a.out_size2 = 1;
+    tr_inner = true;
+  }
   if (!make_plan(a.in, a.out, a.in_stride0, a.in_stride1, a.out_stride0, a.in_size0, a.in_size1,
                  a.out_size0, a.out_size1, a.out_size2, a.out_size3, tr_inner, tr_outer,
                  a.elem_bytes, /*for_unpack=*/false, &plan))
-    return launch_pack_generic(a, stream, name);
+    return launch_pack_generic(original, stream, name);
   plan.args.src = a.in;
   plan.args.dst = a.out;
   plan.args.padding_value = a.padding_value;
