@@ -197,7 +197,14 @@ __device__ __forceinline__ bool locate_block(const MfmaArgs& a, int* tile_row, i
 // row, one 128-bit store (64-bit for a NARROW, i.e. 16-bit, output, rounded to
 // nearest even the way common.h:701-770 does). When accumulating, a fragment's
 // loads are issued before its first add, so their latencies overlap.
-template <int KIND, bool RHS_I4, bool NARROW, int AM, int BN>
+//
+// PAIR_A / PAIR_B: the fragments of that operand were fed in interleaved pairs
+// (2-byte row pieces, see the direct-to-LDS kernel): lane row r of fragments
+// 2p and 2p + 1 is row 64*p + 2*r resp. 64*p + 2*r + 1 of the sub-block. For
+// the columns this means that accumulators e and e + 1 of fragment 2p and of
+// fragment 2p + 1 together are four consecutive j0, so two fragments are
+// written at a time.
+template <int KIND, bool RHS_I4, bool NARROW, int AM, int BN, bool PAIR_A = false, bool PAIR_B = false>
 __device__ __forceinline__ void store_block(const MfmaArgs& a, typename AccType<KIND>::type (&acc)[AM][BN],
                                             int64_t wave_row, int64_t wave_col, int lane) {
   typedef typename AccType<KIND>::scalar scalar_t;
@@ -209,8 +216,8 @@ __device__ __forceinline__ void store_block(const MfmaArgs& a, typename AccType<
   const int32_t M0 = 1 << a.log2_M0, N0 = 1 << a.log2_N0;
   const int64_t total_rows = (int64_t)a.M << a.log2_M0;
   const int64_t total_cols = (int64_t)a.N << a.log2_N0;
-  const int64_t row0 = wave_row + (lane & 31);
-  const int64_t col0 = wave_col + 4 * (lane >> 5);
+  static_assert((!PAIR_A || AM % 2 == 0) && (!PAIR_B || BN % 2 == 0), "pairs of fragments");
+  constexpr int JS = PAIR_B ? 2 : 1;  // rhs fragments written together
   // Byte offset of quad (j, q) from the sub-block's first column tile (the same
   // for every row, and small) and whether the quad lies inside the matrix.
   const int64_t first_col_tile = wave_col >> a.log2_N0;
@@ -221,7 +228,8 @@ __device__ __forceinline__ void store_block(const MfmaArgs& a, typename AccType<
   for (int j = 0; j < BN; ++j)
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      const int64_t col = col0 + 32 * j + 8 * q;
+      const int64_t col = PAIR_B ? wave_col + 8 * (lane >> 5) + 64 * (j >> 1) + 16 * q + 4 * (j & 1)
+                                 : wave_col + 4 * (lane >> 5) + 32 * j + 8 * q;
       col_off[j][q] = (uint32_t)(OUT_BYTES * ((((col >> a.log2_N0) - first_col_tile) << (a.log2_M0 + a.log2_N0)) +
                                               (col & (N0 - 1))));
       if (col < total_cols) col_inside |= 1u << (4 * j + q);
@@ -244,37 +252,57 @@ __device__ __forceinline__ void store_block(const MfmaArgs& a, typename AccType<
   };
 #pragma unroll
   for (int i = 0; i < AM; ++i) {
-    const int64_t row = min(row0 + 32 * i, total_rows - 1);
-    const bool row_inside = row0 + 32 * i < total_rows;
+    const int64_t this_row =
+        wave_row + (PAIR_A ? 64 * (i >> 1) + 2 * (lane & 31) + (i & 1) : 32 * i + (lane & 31));
+    const int64_t row = min(this_row, total_rows - 1);
+    const bool row_inside = this_row < total_rows;
     uint8_t* row_out =
         wave_out + OUT_BYTES * ((row >> a.log2_M0) * a.out_stride0 + ((row & (M0 - 1)) << a.log2_N0));
 #pragma unroll
-    for (int j = 0; j < BN; ++j) {
-      // Pin the fragment where it is until its turn: left alone, the compiler
-      // moves all 256 accumulators to ordinary registers right after the main
-      // loop, and there are not that many.
-      typename AccType<KIND>::type frag = acc[i][j];
-      asm volatile("" : "+a"(frag));
-      quad_t v[4];
+    for (int j0 = 0; j0 < BN; j0 += JS) {
+      // Pin the fragment(s) where they are until their turn: left alone, the
+      // compiler moves all 256 accumulators to ordinary registers right after
+      // the main loop, and there are not that many.
+      typename AccType<KIND>::type frag[JS];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        v[q] = quad_t{frag[4 * q], frag[4 * q + 1], frag[4 * q + 2], frag[4 * q + 3]};
-        if constexpr (RHS_I4) v[q] = v[q] >> 4;
+      for (int s = 0; s < JS; ++s) {
+        frag[s] = acc[i][j0 + s];
+        asm volatile("" : "+a"(frag[s]));
       }
-      if (a.accumulate) {
-        quad_t old[4];
+      quad_t v[JS][4];
+#pragma unroll
+      for (int s = 0; s < JS; ++s)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          old[q] = quad_t{0, 0, 0, 0};
-          if (row_inside && (col_inside >> (4 * j + q) & 1))
-            old[q] = to_float(*(const stored_t*)(row_out + col_off[j][q]));
+          if constexpr (PAIR_B) {
+            v[s][q] = quad_t{frag[0][4 * q + 2 * s], frag[1][4 * q + 2 * s], frag[0][4 * q + 2 * s + 1],
+                             frag[1][4 * q + 2 * s + 1]};
+          } else {
+            v[s][q] = quad_t{frag[s][4 * q], frag[s][4 * q + 1], frag[s][4 * q + 2], frag[s][4 * q + 3]};
+          }
+          if constexpr (RHS_I4) v[s][q] = v[s][q] >> 4;
         }
+      if (a.accumulate) {
+        quad_t old[JS][4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) v[q] += old[q];
+        for (int s = 0; s < JS; ++s)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            old[s][q] = quad_t{0, 0, 0, 0};
+            if (row_inside && (col_inside >> (4 * (j0 + s) + q) & 1))
+              old[s][q] = to_float(*(const stored_t*)(row_out + col_off[j0 + s][q]));
+          }
+#pragma unroll
+        for (int s = 0; s < JS; ++s)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) v[s][q] += old[s][q];
       }
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
-        if (row_inside && (col_inside >> (4 * j + q) & 1)) *(stored_t*)(row_out + col_off[j][q]) = to_stored(v[q]);
+      for (int s = 0; s < JS; ++s)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          if (row_inside && (col_inside >> (4 * (j0 + s) + q) & 1))
+            *(stored_t*)(row_out + col_off[j0 + s][q]) = to_stored(v[s][q]);
       // Keep the fragments apart: hoisting all address arithmetic and
       // accumulator reads to the top costs more registers than there are.
       __builtin_amdgcn_sched_barrier(0);
@@ -544,6 +572,9 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   constexpr int STAGE_PIECES = A_PIECES + B_PIECES;
   constexpr int AHEAD = STAGES - 1;  // chunks in flight ahead of the one being multiplied
   static_assert(STAGES >= 4, "ring depth");
+  // 2-byte row pieces: an operand with an even number of fragments per
+  // wavefront is fed in interleaved pairs of fragments (see the layouts below).
+  constexpr bool PAIR_A = G == 2 && AM % 2 == 0, PAIR_B = G == 2 && BN % 2 == 0;
   // Load instructions per wavefront and chunk (64 lanes x 16 bytes each), each
   // with its own per-lane offset.
   constexpr int A_LOADS = A_PIECES / 256, B_LOADS = B_PIECES / 256;
@@ -592,8 +623,25 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   //     MFMA operand of lane 32*h + r for K-step kk is elements d = 0 .. 16/G - 1,
   //     each read linear in the lane number (4-byte pieces: two paired dword
   //     reads; 8-byte: two 64-bit reads; 2-byte: eight 16-bit reads, which
-  //     makes those layouts LDS-instruction bound). K is permuted inside a
+  //     makes that layout LDS-instruction bound). K is permuted inside a
   //     chunk, identically for lhs and rhs.
+  //   G == 2, fragments in pairs (an even number of them per wavefront): 16-bit
+  //     reads deliver half of what the LDS can, so a lane reads dwords, i.e. two
+  //     adjacent rows of one k step, and gives the low half to fragment 2p, the
+  //     high half to fragment 2p + 1: row r of those fragments is row 2*r resp.
+  //     2*r + 1 of the pair's 64 rows (the epilogue undoes it). Slot 64*m + l
+  //     holds rows 8*g .. 8*g + 7 (g = l & 7) of pair m >> 2 at k step
+  //     16*kk + 8*h + 4*(m & 1) + (l >> 4) of the chunk (kk = (m >> 1) & 1,
+  //     h = (l >> 3) & 1), the same k steps per (K-step, lane half) as in the
+  //     unpaired layout, so the two can be mixed between lhs and rhs. Dword
+  //     64*d + 32*h + r of a (pair, K-step) is then rows 2*r, 2*r + 1 at the
+  //     lane's d-th k step: eight dword reads linear in the lane number (four
+  //     two-address instructions) and eight byte permutes per two fragments.
+  //     (Tried: lanes arranged so that four consecutive ones load four
+  //     consecutive k steps of one row group, i.e. one cache line instead of
+  //     two for M0 = 16 or four for M0 = 8, with an xor spreading the row groups
+  //     over the banks. The reads then need eight separate addresses: 8x8x2
+  //     int8 tiles went from 114 to 100 us per 4096^3, 16x16x2 from 83 to 89.)
   //   int4 rhs: slot 64*f + 32*h + r holds nibbles 32*h .. 32*h + 31 of row r of
   //     fragment f: lane 32*h + r reads that slot once per chunk and widens its
   //     first 8 bytes for K-step 0, its last 8 for K-step 1. The lhs columns are
@@ -628,19 +676,32 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
     }
   } else {
     constexpr int R = 16 / G;  // rows per 16-byte piece
-    const int g = lane % (2 * G), k1 = (16 / G) * ((lane / (2 * G)) & 1) + lane / (4 * G);
+    // Row group and k step of the chunk of this lane's piece in load t (the
+    // wavefront's share of the k steps included).
+    auto piece_of = [&](bool paired, int t, int* row, int* k1) {
+      if (paired) {
+        *row = 64 * t + 8 * (lane & 7);
+        *k1 = 16 * (wave >> 1) + 8 * ((lane >> 3) & 1) + 4 * (wave & 1) + (lane >> 4);
+      } else {
+        *row = 32 * (2 * t + (wave >> 1)) + R * (lane % (2 * G));
+        *k1 = (32 / G) * (wave & 1) + (16 / G) * ((lane / (2 * G)) & 1) + lane / (4 * G);
+      }
+    };
 #pragma unroll
-    for (int t = 0; t < A_LOADS; ++t)
-      a_off[t] = (uint32_t)(row_offset(first_row + 32 * (2 * t + (wave >> 1)) + R * g, total_rows - R, first_row,
-                                       a.log2_M0, a.lhs_stride_bytes, a.lhs_rb) + k1 * lhs_kstep);
+    for (int t = 0; t < A_LOADS; ++t) {
+      int row, k1;
+      piece_of(PAIR_A, t, &row, &k1);
+      a_off[t] = (uint32_t)(row_offset(first_row + row, total_rows - R, first_row, a.log2_M0, a.lhs_stride_bytes,
+                                       a.lhs_rb) + k1 * lhs_kstep);
+    }
 #pragma unroll
-    for (int t = 0; t < B_LOADS; ++t)
-      b_off[t] = (uint32_t)(row_offset(first_col + 32 * (2 * t + (wave >> 1)) + R * g, total_cols - R, first_col,
-                                       a.log2_N0, a.rhs_stride_bytes, a.rhs_rb) + k1 * rhs_kstep);
+    for (int t = 0; t < B_LOADS; ++t) {
+      int row, k1;
+      piece_of(PAIR_B, t, &row, &k1);
+      b_off[t] = (uint32_t)(row_offset(first_col + row, total_cols - R, first_col, a.log2_N0, a.rhs_stride_bytes,
+                                       a.rhs_rb) + k1 * rhs_kstep);
+    }
   }
-  // G < 16: this wavefront's loads all belong to K-step wave & 1.
-  const int64_t lhs_wave_bytes = G < 16 ? (32 / G) * (wave & 1) * lhs_kstep : 0;
-  const int64_t rhs_wave_bytes = G < 16 ? (32 / G) * (wave & 1) * rhs_kstep : 0;
 
   acc_t acc[AM][BN];
 #pragma unroll
@@ -664,8 +725,8 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   auto issue_chunk = [&](int kc) {
     const int idx = min(kc, last_chunk);
     const uint32_t stage_off = (uint32_t)(kc % STAGES) * (STAGE_PIECES * 16);
-    const uint8_t* la = lhs_base + idx * lhs_chunk_bytes + lhs_wave_bytes;
-    const uint8_t* lb = rhs_base + idx * rhs_chunk_bytes + rhs_wave_bytes;
+    const uint8_t* la = lhs_base + idx * lhs_chunk_bytes;
+    const uint8_t* lb = rhs_base + idx * rhs_chunk_bytes;
 #pragma unroll
     for (int n = 0; n < LOADS; ++n) issue_load(n, stage_off, la, lb);
   };
@@ -699,6 +760,18 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
       return make_uint4(gather_dword(first, 0), gather_dword(first, 1), gather_dword(first, 2), gather_dword(first, 3));
     }
   };
+  // Paired fragments: dwords 2*part and 2*part + 1 of the lane's eight for
+  // (pair, K-step), split into dword `part` of the even and of the odd fragment.
+  auto set_dword = [](uint4& v, int part, uint32_t w) {
+    if (part == 0) v.x = w; else if (part == 1) v.y = w; else if (part == 2) v.z = w; else v.w = w;
+  };
+  auto read_pair_part = [](const uint8_t* first, int part) -> uint2 {
+    return make_uint2(*(const uint32_t*)(first + 512 * part), *(const uint32_t*)(first + 512 * part + 256));
+  };
+  auto split_pair_part = [&](uint2 w, int part, uint4& even, uint4& odd) {
+    set_dword(even, part, __builtin_amdgcn_perm(w.y, w.x, 0x05040100u));
+    set_dword(odd, part, __builtin_amdgcn_perm(w.y, w.x, 0x07060302u));
+  };
   const int frag_a0 = wave_m * AM, frag_b0 = wave_n * BN;
 
   // Loop-carried, wavefront-uniform state: where the next chunk to load comes
@@ -707,8 +780,8 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   // chunk number (64-bit multiplies on the scalar unit, in front of the step's
   // first MFMA).
   constexpr uint32_t STAGE_BYTES = STAGE_PIECES * 16, RING_BYTES = STAGES * STAGE_BYTES;
-  const uint8_t* load_a = lhs_base + min(AHEAD, last_chunk) * lhs_chunk_bytes + lhs_wave_bytes;
-  const uint8_t* load_b = rhs_base + min(AHEAD, last_chunk) * rhs_chunk_bytes + rhs_wave_bytes;
+  const uint8_t* load_a = lhs_base + min(AHEAD, last_chunk) * lhs_chunk_bytes;
+  const uint8_t* load_b = rhs_base + min(AHEAD, last_chunk) * rhs_chunk_bytes;
   int load_chunk = AHEAD;
   uint32_t load_stage_off = AHEAD * STAGE_BYTES % RING_BYTES;
   uint32_t read_stage_off = STAGE_BYTES;
@@ -720,6 +793,7 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   const uint8_t* ring_bytes =
       (const uint8_t*)ring + (ROWS16 ? 16 * (64 * ((lane & 31) >> 4) + 16 * (lane >> 5) + (lane & 15))
                                      : (G == 16 ? 16 : G) * lane);
+  const uint32_t pair_a_lane = PAIR_A ? 2 * lane : 0, pair_b_lane = PAIR_B ? 2 * lane : 0;  // dwords, not 16-bit elements
   constexpr int KK16 = ROWS16 ? 32 : 64;
 
   // One pipeline step for the chunk whose fragments are in `cur`:
@@ -745,12 +819,40 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
     // fragments, then the lhs fragments. An int4 rhs fragment is read once, raw,
     // for both K-steps (first), and widened after the last read has been issued.
     constexpr int B_UNITS = RHS_I4 ? BN : 0;
-    constexpr int READS = RHS_I4 ? BN + 2 * AM : 2 * (AM + BN) * PARTS;
+    constexpr int UNITS_A = AM * (PAIR_A ? 2 : PARTS), UNITS_B = BN * (PAIR_B ? 2 : PARTS);  // per K-step
+    constexpr int READS = RHS_I4 ? BN + 2 * AM : 2 * (UNITS_A + UNITS_B);
     constexpr int LEAD = MFMAS >= 16 ? 4 : (MFMAS >= 8 ? 2 : 0);   // MFMAs ahead of the barrier
     constexpr int TAIL_FREE = MFMAS >= 8 ? MFMAS / 4 : (RHS_I4 ? 1 : 0);  // MFMAs after the last read
     constexpr int SLOTS = MFMAS - LEAD - TAIL_FREE;                // MFMAs that carry memory work
     static_assert(SLOTS >= 1, "no room for the memory instructions");
     static_assert(!RHS_I4 || TAIL_FREE >= 1, "nowhere to widen");
+    // Paired fragments: the dwords of a read unit are split this many MFMAs
+    // after the read was issued (a wavefront issues in order: splitting right
+    // away would stall it, MFMAs included, for the LDS latency of every unit).
+    constexpr int SPLIT_DELAY = TAIL_FREE < 3 ? TAIL_FREE : 3;
+    uint2 raw_pair[(PAIR_A || PAIR_B) ? READS : 1];
+    // Where read unit u of the next step's fragments goes.
+    auto unit_of = [&](int u, bool* is_b, bool* paired, int* kk, int* y) {
+      *kk = u / (UNITS_A + UNITS_B);
+      const int x = u % (UNITS_A + UNITS_B);
+      *is_b = x < UNITS_B;
+      *paired = *is_b ? PAIR_B : PAIR_A;
+      *y = *is_b ? x : x - UNITS_B;
+    };
+    auto split_units_of = [&](int read_slot) {
+      if constexpr (PAIR_A || PAIR_B) {
+        if (read_slot < 0 || read_slot >= SLOTS) return;
+#pragma unroll
+        for (int u = read_slot * READS / SLOTS; u < (read_slot + 1) * READS / SLOTS; ++u) {
+          bool is_b, paired;
+          int kk, y;
+          unit_of(u, &is_b, &paired, &kk, &y);
+          if (!paired) continue;
+          uint4(*nxt)[2] = is_b ? nxt_b : nxt_a;
+          split_pair_part(raw_pair[u], y % 4, nxt[2 * (y / 4)][kk], nxt[2 * (y / 4) + 1][kk]);
+        }
+      }
+    };
     auto multiply = [&](int m) {
       const int kk = m / (AM * BN * SUB), sub = (m / (AM * BN)) % SUB, i = (m % (AM * BN)) / BN, j = m % BN;
       acc[i][j] = mfma<KIND>(cur_b[j][kk], cur_a[i][kk], acc[i][j], sub);
@@ -760,8 +862,8 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
     __builtin_amdgcn_sched_barrier(0);
     wait_loads_but<LOADS*(AHEAD - 2)>();
     __builtin_amdgcn_s_barrier();
-    const uint8_t* read_a = ring_bytes + read_stage_off + frag_a_off;
-    const uint8_t* read_b = ring_bytes + read_stage_off + frag_b_off;
+    const uint8_t* read_a = ring_bytes + read_stage_off + frag_a_off + pair_a_lane;
+    const uint8_t* read_b = ring_bytes + read_stage_off + frag_b_off + pair_b_lane;
     uint4 raw_b[RHS_I4 ? BN : 1];
 #pragma unroll
     for (int m = LEAD; m < MFMAS; ++m) {
@@ -781,11 +883,17 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
               nxt_a[i][kk] = *(const uint4*)(read_a + (128 * i + KK16 * kk) * 16);
             }
           } else {
-            const int f = u / PARTS, part = u % PARTS;
-            const int kk = f / (AM + BN), e = f % (AM + BN);
-            uint4& dst = e < BN ? nxt_b[e][kk] : nxt_a[e - BN][kk];
-            const uint8_t* src = e < BN ? read_b : read_a;
-            const int frag = e < BN ? e : e - BN;
+            bool is_b, paired;
+            int kk, y;
+            unit_of(u, &is_b, &paired, &kk, &y);
+            const uint8_t* src = is_b ? read_b : read_a;
+            uint4(*nxt)[2] = is_b ? nxt_b : nxt_a;
+            if (paired) {
+              raw_pair[u] = read_pair_part(src + 4096 * (y / 4) + 2048 * kk, y % 4);
+              continue;
+            }
+            const int frag = y / PARTS, part = y % PARTS;
+            uint4& dst = nxt[frag][kk];
             if constexpr (G == 16) {
               dst = *(const uint4*)(src + (128 * frag + KK16 * kk) * 16);
             } else {
@@ -793,6 +901,12 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
               if constexpr (G == 2) {
                 const uint32_t w = gather_dword(first, part);
                 if (part == 0) dst.x = w; else if (part == 1) dst.y = w; else if (part == 2) dst.z = w; else dst.w = w;
+              } else if constexpr (G == 8) {
+                // One 64-bit read (two dword reads of adjacent addresses, which
+                // is what the compiler makes of 4-byte aligned accesses, collide
+                // on the banks: lanes are 8 bytes apart).
+                const uint2 w = *(const uint2*)(first + part * 512);
+                if (part == 0) { dst.x = w.x; dst.y = w.y; } else { dst.z = w.x; dst.w = w.y; }
               } else {
                 if (part == 0) { dst.x = gather_dword(first, 0); dst.y = gather_dword(first, 1); }
                 else { dst.z = gather_dword(first, 2); dst.w = gather_dword(first, 3); }
@@ -809,6 +923,7 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
           nxt_b[j][kk] = widen_i4_times16(kk ? make_uint2(raw_b[j].z, raw_b[j].w) : make_uint2(raw_b[j].x, raw_b[j].y));
         }
       }
+      split_units_of(slot - SPLIT_DELAY);
       multiply(m);
       if (m == MFMAS - 1) {
         // Advance the running state (clamped at the last chunk: the loads
@@ -831,9 +946,32 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
 #pragma unroll
   for (int kk = 0; kk < 2; ++kk) {
 #pragma unroll
-    for (int j = 0; j < BN; ++j) pb[j][kk] = read_frag(A_PIECES, frag_b0 + j, kk);
+    for (int j = 0; j < BN; ++j) {
+      if constexpr (PAIR_B) {
+        if (j % 2 == 0) {
 #pragma unroll
-    for (int i = 0; i < AM; ++i) pa[i][kk] = read_frag(0, frag_a0 + i, kk);
+          for (int part = 0; part < 4; ++part)
+            split_pair_part(
+                read_pair_part((const uint8_t*)(ring + A_PIECES) + 2048 * (frag_b0 + j) + 2048 * kk + 4 * lane, part),
+                part, pb[j][kk], pb[j + 1][kk]);
+        }
+      } else {
+        pb[j][kk] = read_frag(A_PIECES, frag_b0 + j, kk);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < AM; ++i) {
+      if constexpr (PAIR_A) {
+        if (i % 2 == 0) {
+#pragma unroll
+          for (int part = 0; part < 4; ++part)
+            split_pair_part(read_pair_part((const uint8_t*)ring + 2048 * (frag_a0 + i) + 2048 * kk + 4 * lane, part),
+                            part, pa[i][kk], pa[i + 1][kk]);
+        }
+      } else {
+        pa[i][kk] = read_frag(0, frag_a0 + i, kk);
+      }
+    }
   }
   int kc = 0;
   for (; kc + 1 < chunks; kc += 2) {
@@ -844,8 +982,8 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   // No load may still be writing LDS when the workgroup's allocation is freed.
   wait_loads_but<0>();
 
-  store_block<KIND, RHS_I4, NARROW, AM, BN>(a, acc, first_row + wave_m * (32 * AM),
-                                            first_col + wave_n * (32 * BN), lane);
+  store_block<KIND, RHS_I4, NARROW, AM, BN, PAIR_A, PAIR_B>(a, acc, first_row + wave_m * (32 * AM),
+                                                            first_col + wave_n * (32 * BN), lane);
 }
 
 // Whether the direct-to-LDS kernel covers the problem: K ends on a chunk

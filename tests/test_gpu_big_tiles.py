@@ -36,7 +36,8 @@ def run_case(gpu_lib, flags, M, N, K, M0, N0, K0, expect_kernel, lhs_pad=0, rhs_
         if kind in (abi.MMT4D_TYPE_S8S8S32, abi.MMT4D_TYPE_S8S4S32):
             return torch.randint(-128, 128, (off + n_tiles * stride,), dtype=torch.int8, device="cuda", generator=g)
         dt = {abi.MMT4D_TYPE_F16F16F32: torch.float16, abi.MMT4D_TYPE_BF16BF16F32: torch.bfloat16,
-              abi.MMT4D_TYPE_F32F32F32: torch.float32}[kind]
+              abi.MMT4D_TYPE_F32F32F32: torch.float32, abi.MMT4D_TYPE_F16F16F16: torch.float16,
+              abi.MMT4D_TYPE_BF16BF16BF16: torch.bfloat16}[kind]
         return (torch.randn(off + n_tiles * stride, device="cuda", generator=g) / 8).to(dt)
 
     lhs = operand(M, lhs_stride, lo, M0)
@@ -47,11 +48,17 @@ def run_case(gpu_lib, flags, M, N, K, M0, N0, K0, expect_kernel, lhs_pad=0, rhs_
     else:
         rhs = operand(N, rhs_stride, ro, N0)
     is_int = kind in (abi.MMT4D_TYPE_S8S8S32, abi.MMT4D_TYPE_S8S4S32)
-    out_dtype = torch.int32 if is_int else torch.float32
+    # 16-bit outputs reach the matrix pipe only with the roundings between k steps skipped; one final rounding then.
+    narrow = {abi.MMT4D_TYPE_F16F16F16: (torch.float16, 2.0 ** -10), abi.MMT4D_TYPE_BF16BF16BF16: (torch.bfloat16, 2.0 ** -7)}
+    out_ulp = narrow[kind][1] if kind in narrow else 0.0
+    if kind in narrow:
+        flags |= abi.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS
     if is_int:
         out = torch.randint(-1000, 1000, (oo + M * out_stride,), dtype=torch.int32, device="cuda", generator=g)
     else:
         out = torch.randn(oo + M * out_stride, device="cuda", generator=g)
+        if kind in narrow:
+            out = out.to(narrow[kind][0])
     before = out.clone()
     p = mm_params(lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), M, N, K, M0, N0, K0,
                   flags | (abi.MMT4D_ACCUMULATE if accumulate else 0), lhs_off=lo, rhs_off=ro, out_off=oo,
@@ -81,7 +88,7 @@ def run_case(gpu_lib, flags, M, N, K, M0, N0, K0, expect_kernel, lhs_pad=0, rhs_
         assert torch.equal(got.long(), ref.long())
     else:
         rms = ref.pow(2).mean().sqrt()
-        assert bool(((got.double() - ref).abs() <= REL_TOL * torch.maximum(ref.abs(), rms)).all())
+        assert bool(((got.double() - ref).abs() <= (REL_TOL + out_ulp) * torch.maximum(ref.abs(), rms)).all())
     # Nothing outside the output tiles was written: the gaps between tile rows and the prefix.
     if out_pad:
         gaps = out[oo:oo + M * out_stride].view(M, out_stride)[:, N * M0 * N0:]
@@ -118,7 +125,8 @@ def test_s8s8s32_ragged_128(gpu_lib, M, N):
 
 @pytest.mark.parametrize("flags,M0,N0,K0,K", [(abi.MMT4D_TYPE_F16F16F32, 16, 16, 16, 10), (abi.MMT4D_TYPE_BF16BF16F32, 16, 16, 8, 13),
                                               (abi.MMT4D_TYPE_F16F16F32, 8, 8, 2, 48), (abi.MMT4D_TYPE_F32F32F32, 16, 16, 4, 11),
-                                              (abi.MMT4D_TYPE_F32F32F32, 8, 8, 1, 33)])
+                                              (abi.MMT4D_TYPE_F32F32F32, 8, 8, 1, 33), (abi.MMT4D_TYPE_F16F16F16, 16, 16, 16, 6),
+                                              (abi.MMT4D_TYPE_BF16BF16BF16, 8, 16, 2, 40)])
 def test_float_types_ragged_256(gpu_lib, flags, M0, N0, K0, K):
     M, N = 3608 // M0 + 1, 3704 // N0 + 1
     run_case(gpu_lib, flags, M, N, K, M0, N0, K0, "mmt4d_mfma_256x256", accumulate=True, out_pad=16, seed=K)
@@ -157,6 +165,20 @@ def test_narrow_and_8_byte_row_pieces(gpu_lib, flags, M0, N0, K0, K):
     # the smallest block tile, strided operands with offsets (all multiples of 16 bytes)
     run_case(gpu_lib, flags, 72 // M0, 88 // N0, K, M0, N0, K0, "mmt4d_mfma_64x64", lhs_pad=32, rhs_pad=16,
              offsets=(16, 32, 4), seed=K0)
+
+
+# 2-byte row pieces feed the matrix pipe in interleaved pairs of fragments wherever a wavefront owns an even number of
+# fragments of an operand (rows 2r / 2r+1 of 64 from one dword), which the epilogue has to undo: every block tile, with
+# the lhs paired and the rhs not (128x64), ragged edges that cut pairs apart, accumulation and padded output rows.
+@pytest.mark.parametrize("flags,M0,N0,K0,K", [(abi.MMT4D_TYPE_S8S8S32, 16, 16, 2, 64), (abi.MMT4D_TYPE_S8S8S32, 8, 8, 2, 32),
+                                              (abi.MMT4D_TYPE_F16F16F32, 16, 16, 1, 96), (abi.MMT4D_TYPE_BF16BF16F32, 8, 16, 1, 32)])
+def test_two_byte_row_pieces_on_every_block_tile(gpu_lib, flags, M0, N0, K0, K):
+    n_cols = 14300 // N0 * N0
+    run_case(gpu_lib, flags, 504 // M0, n_cols // N0, K, M0, N0, K0, "mmt4d_mfma_256x128", accumulate=True, out_pad=8, seed=K)
+    run_case(gpu_lib, flags, 120 // M0, n_cols // N0, K, M0, N0, K0, "mmt4d_mfma_128x64", seed=K + 1)
+    run_case(gpu_lib, flags, 1608 // M0, 1912 // N0, K, M0, N0, K0, "mmt4d_mfma_128x128", accumulate=True, seed=K + 2)
+    run_case(gpu_lib, flags, 3608 // M0 + 1, 3704 // N0 + 1, K, M0, N0, K0, "mmt4d_mfma_256x256", lhs_pad=32, rhs_pad=16,
+             out_pad=12, offsets=(16, 32, 4), seed=K + 3)
 
 
 def test_narrow_row_pieces_fall_back_when_the_direct_kernel_cannot_run(gpu_lib):
