@@ -12,10 +12,12 @@
 // Two kernels share this tiling and the epilogue:
 //   mmt4d_mfma_direct_kernel (the fast path): operands go global memory ->
 //     LDS directly, 16 contiguous bytes per lane, through a ring of LDS stages
-//     filled several chunks ahead; needs K to end on a chunk boundary and
-//     16-byte aligned operand rows.
-//   mmt4d_mfma_kernel (everything else the plan admits: ragged K, 4-byte
-//     aligned operands, narrow tiles): global -> registers (issued two chunks
+//     filled several chunks ahead; needs 16-byte aligned operand rows and at
+//     least one full chunk of K (a K that ends inside a chunk is handled by
+//     overlapping the last chunk with the one before it).
+//   mmt4d_mfma_kernel (everything else the plan admits: 4-byte aligned
+//     operands, narrow tiles, less than a chunk of K, an int4 rhs whose K ends
+//     inside a chunk): global -> registers (issued two chunks
 //     ahead) -> LDS -> registers (read one chunk ahead) -> MFMA.
 // In both, LDS holds the operands fragment-major, so that a wavefront fetches
 // a 32-row x 32-byte MFMA operand with conflict-free reads that are linear in
@@ -711,8 +713,18 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
 
-  const int chunks = a.chunks;  // all full
+  // K may end inside the last chunk (not with an int4 rhs). That chunk is then
+  // loaded from where a full chunk ends at K, so it overlaps the chunk before
+  // it and every load stays inside the operands, and the overlap, i.e. the
+  // first `cut_bytes` of its 64 bytes per row, is zeroed in the fragments of
+  // both operands (0 * 0 adds nothing, whatever the data).
+  const int chunks = a.chunks;
   const int last_chunk = chunks - 1;
+  const int32_t cut_bytes = RHS_I4 ? 0 : (int32_t)((64 - (((int64_t)a.K << a.log2_lhs_rb) & 63)) & 63);
+  const int64_t lhs_last_base = a.K * lhs_kstep - lhs_chunk_bytes;
+  const int64_t rhs_last_base = a.K * rhs_kstep - rhs_chunk_bytes;
+  const int64_t lhs_last_advance = lhs_last_base - (last_chunk - 1) * lhs_chunk_bytes;
+  const int64_t rhs_last_advance = rhs_last_base - (last_chunk - 1) * rhs_chunk_bytes;
 
   // Load number `n` (compile-time after unrolling) of the chunk whose operand
   // bases are la / lb, into the stage at LDS byte offset `stage_off`.
@@ -725,8 +737,8 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   auto issue_chunk = [&](int kc) {
     const int idx = min(kc, last_chunk);
     const uint32_t stage_off = (uint32_t)(kc % STAGES) * (STAGE_PIECES * 16);
-    const uint8_t* la = lhs_base + idx * lhs_chunk_bytes;
-    const uint8_t* lb = rhs_base + idx * rhs_chunk_bytes;
+    const uint8_t* la = lhs_base + (idx == last_chunk ? lhs_last_base : idx * lhs_chunk_bytes);
+    const uint8_t* lb = rhs_base + (idx == last_chunk ? rhs_last_base : idx * rhs_chunk_bytes);
 #pragma unroll
     for (int n = 0; n < LOADS; ++n) issue_load(n, stage_off, la, lb);
   };
@@ -780,8 +792,8 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   // chunk number (64-bit multiplies on the scalar unit, in front of the step's
   // first MFMA).
   constexpr uint32_t STAGE_BYTES = STAGE_PIECES * 16, RING_BYTES = STAGES * STAGE_BYTES;
-  const uint8_t* load_a = lhs_base + min(AHEAD, last_chunk) * lhs_chunk_bytes;
-  const uint8_t* load_b = rhs_base + min(AHEAD, last_chunk) * rhs_chunk_bytes;
+  const uint8_t* load_a = lhs_base + (AHEAD >= last_chunk ? lhs_last_base : AHEAD * lhs_chunk_bytes);
+  const uint8_t* load_b = rhs_base + (AHEAD >= last_chunk ? rhs_last_base : AHEAD * rhs_chunk_bytes);
   int load_chunk = AHEAD;
   uint32_t load_stage_off = AHEAD * STAGE_BYTES % RING_BYTES;
   uint32_t read_stage_off = STAGE_BYTES;
@@ -862,6 +874,8 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
     __builtin_amdgcn_sched_barrier(0);
     wait_loads_but<LOADS*(AHEAD - 2)>();
     __builtin_amdgcn_s_barrier();
+    // The fragments read during this step are those of chunk load_chunk - AHEAD + 1.
+    const bool cut_next = cut_bytes != 0 && load_chunk - AHEAD + 1 == last_chunk;
     const uint8_t* read_a = ring_bytes + read_stage_off + frag_a_off + pair_a_lane;
     const uint8_t* read_b = ring_bytes + read_stage_off + frag_b_off + pair_b_lane;
     uint4 raw_b[RHS_I4 ? BN : 1];
@@ -928,14 +942,36 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
       if (m == MFMAS - 1) {
         // Advance the running state (clamped at the last chunk: the loads
         // issued beyond it are redundant, their stages are never read).
-        const bool more = load_chunk < last_chunk;
-        load_a += more ? lhs_chunk_bytes : 0;
-        load_b += more ? rhs_chunk_bytes : 0;
+        const bool more = load_chunk < last_chunk, to_last = load_chunk + 1 == last_chunk;
+        load_a += more ? (to_last ? lhs_last_advance : lhs_chunk_bytes) : 0;
+        load_b += more ? (to_last ? rhs_last_advance : rhs_chunk_bytes) : 0;
         ++load_chunk;
         load_stage_off = load_stage_off + STAGE_BYTES == RING_BYTES ? 0 : load_stage_off + STAGE_BYTES;
         read_stage_off = read_stage_off + STAGE_BYTES == RING_BYTES ? 0 : read_stage_off + STAGE_BYTES;
       }
       __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (!RHS_I4) {
+      if (cut_next) {
+        // Lane half h of K-step kk holds bytes 32*kk + 16*h .. + 15 of the chunk's
+        // 64 bytes per row, in ascending order of k in every layout above.
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+          const int cut = min(max(cut_bytes - 32 * kk - 16 * (lane >> 5), 0), 16);
+          uint32_t keep[4];
+#pragma unroll
+          for (int w = 0; w < 4; ++w)
+            keep[w] = cut >= 4 * w + 4 ? 0u : (cut <= 4 * w ? 0xFFFFFFFFu : 0xFFFFFFFFu << (8 * (cut - 4 * w)));
+#pragma unroll
+          for (int i = 0; i < AM; ++i) {
+            nxt_a[i][kk].x &= keep[0]; nxt_a[i][kk].y &= keep[1]; nxt_a[i][kk].z &= keep[2]; nxt_a[i][kk].w &= keep[3];
+          }
+#pragma unroll
+          for (int j = 0; j < BN; ++j) {
+            nxt_b[j][kk].x &= keep[0]; nxt_b[j][kk].y &= keep[1]; nxt_b[j][kk].z &= keep[2]; nxt_b[j][kk].w &= keep[3];
+          }
+        }
+      }
     }
   };
 
@@ -986,12 +1022,14 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
                                                             first_col + wave_n * (32 * BN), lane);
 }
 
-// Whether the direct-to-LDS kernel covers the problem: K ends on a chunk
-// boundary and every lane can load 16 contiguous bytes (4-byte row pieces 4
-// rows at a time, an int4 rhs in pieces of 32 nibbles).
+// Whether the direct-to-LDS kernel covers the problem: every lane can load 16
+// contiguous bytes (4-byte row pieces 4 rows at a time, an int4 rhs in pieces
+// of 32 nibbles), and K is long enough.
 template <bool RHS_I4, int G>
 bool direct_covers(const MfmaArgs& m) {
-  if (((int64_t)m.K * m.lhs_rb) % 64 != 0) return false;
+  // K ending inside a chunk: not with an int4 rhs, and one full chunk at least.
+  const int64_t row_bytes = (int64_t)m.K * m.lhs_rb;
+  if (row_bytes % 64 != 0 && (RHS_I4 || row_bytes < 64)) return false;
   if (RHS_I4) return m.rhs_rb >= 16 && (uintptr_t)m.rhs % 16 == 0 && m.rhs_stride_bytes % 16 == 0;
   if (G == 16) return true;
   // 16 / G rows of one k step make up a lane's 16 bytes: tiles at least that tall.

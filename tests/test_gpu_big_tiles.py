@@ -182,9 +182,44 @@ def test_two_byte_row_pieces_on_every_block_tile(gpu_lib, flags, M0, N0, K0, K):
 
 
 def test_narrow_row_pieces_fall_back_when_the_direct_kernel_cannot_run(gpu_lib):
-    # K not a multiple of the chunk, or rows not 16-byte aligned: the generic kernel, still exact.
-    run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, 9, 11, 33, 16, 16, 2, "mmt4d_generic", accumulate=True)
+    # Less than one 64-byte chunk of K, or rows not 16-byte aligned: the generic kernel, still exact.
+    run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, 9, 11, 31, 16, 16, 2, "mmt4d_generic", accumulate=True)
     run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, 9, 11, 32, 16, 16, 2, "mmt4d_generic", lhs_pad=4)
+    run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, 9, 11, 33, 16, 16, 2, "mmt4d_mfma_64x64", accumulate=True)
+
+
+# K ending inside a 64-byte chunk on the direct-to-LDS kernel: the last chunk overlaps the one before it and the
+# overlap is zeroed in the fragments. Every row piece size, cuts at every granularity (an odd number of k steps,
+# cuts inside a lane's 16 bytes and at 16- and 32-byte boundaries), one chunk plus a bit, every block tile.
+@pytest.mark.parametrize("flags,M0,N0,K0,Ks", [
+    (abi.MMT4D_TYPE_S8S8S32, 8, 8, 4, (17, 21, 24, 27, 31, 45)), (abi.MMT4D_TYPE_S8S8S32, 16, 16, 2, (33, 40, 47, 49, 63, 95)),
+    (abi.MMT4D_TYPE_S8S8S32, 8, 8, 8, (9, 11, 13, 22)), (abi.MMT4D_TYPE_S8S8S32, 16, 16, 16, (5, 6, 7, 9)),
+    (abi.MMT4D_TYPE_S8S8S32, 16, 8, 32, (3, 5)), (abi.MMT4D_TYPE_F16F16F32, 16, 16, 1, (33, 50, 77)),
+    (abi.MMT4D_TYPE_F16F16F32, 16, 16, 16, (3, 5)), (abi.MMT4D_TYPE_BF16BF16F32, 8, 8, 4, (9, 15, 20)),
+    (abi.MMT4D_TYPE_BF16BF16F32, 16, 16, 2, (17, 30)), (abi.MMT4D_TYPE_F32F32F32, 16, 16, 4, (5, 6, 7)),
+    (abi.MMT4D_TYPE_F32F32F32, 8, 8, 1, (17, 33)), (abi.MMT4D_TYPE_F32F32F32, 8, 16, 2, (9, 13))])
+def test_direct_kernel_with_K_ending_inside_a_chunk(gpu_lib, flags, M0, N0, K0, Ks):
+    n_cols = 14300 // N0 * N0
+    for n, K in enumerate(Ks):
+        tile = n % 4
+        if tile == 0:
+            run_case(gpu_lib, flags, 3608 // M0 + 1, 3704 // N0 + 1, K, M0, N0, K0, "mmt4d_mfma_256x256", accumulate=True,
+                     out_pad=16, seed=K)
+        elif tile == 1:
+            run_case(gpu_lib, flags, 504 // M0, n_cols // N0, K, M0, N0, K0, "mmt4d_mfma_256x128", lhs_pad=32, rhs_pad=16,
+                     offsets=(16, 32, 4), seed=K)
+        elif tile == 2:
+            run_case(gpu_lib, flags, 120 // M0, n_cols // N0, K, M0, N0, K0, "mmt4d_mfma_128x64", accumulate=True, seed=K)
+        else:
+            run_case(gpu_lib, flags, 1608 // M0, 1912 // N0, K, M0, N0, K0, "mmt4d_mfma_128x128", seed=K)
+        run_case(gpu_lib, flags, 72 // M0, 88 // N0, K, M0, N0, K0, "mmt4d_mfma_64x64", accumulate=True, seed=K + 100)
+
+
+def test_ragged_K_on_the_register_staged_kernel(gpu_lib):
+    # 4-byte aligned rows (not 16): the register-staged kernel with its zero-filling tail step.
+    run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, 451, 463, 37, 8, 8, 4, "mmt4d_mfma_256x256", lhs_pad=4, rhs_pad=12,
+             out_pad=4, offsets=(4, 20, 4), accumulate=True, seed=5)
+    run_case(gpu_lib, abi.MMT4D_TYPE_BF16BF16F32, 100, 119, 19, 16, 16, 2, "mmt4d_mfma_128x128", lhs_pad=2, rhs_pad=6, seed=6)
 
 
 # The 64x128 block tile of the int4 rhs, picked for a few dozen lhs rows against many rhs rows.
