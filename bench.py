@@ -217,6 +217,23 @@ def _also(torch, lib, abi, synth, steps, warmup):
             "kernel": lib.iree_uk_mi355x_last_kernel().decode(), "ms": round(ms, 5),
             "value": round(nbytes / ms / 1e6, 1), "unit": "GB/s",
             "frac_of_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+    # The same rhs bytes read as the narrow tiles an x86-64 target picks for a
+    # matrix-vector product (bf16 1x16x2, mmt4d_x86_64_tiles.inl): 4-byte row
+    # pieces, which no MFMA operand can be loaded from directly.
+    lhs = f16_operand(4, 1, 4096, 1.0, bf16=True)
+    outs = torch.zeros(896 * 16, dtype=torch.float32, device="cuda")
+    ps = [_mmt4d_params(abi, lhs.data_ptr(), r.data_ptr(), outs.data_ptr(), 1, 896, 2048, 1, 16, 2,
+                        abi.MMT4D_TYPE_BF16BF16F32) for r in rhs_set]
+    state = {"i": 0}
+
+    def step_narrow():
+        lib.iree_uk_mmt4d_p(C.byref(ps[state["i"] % 3]))
+        state["i"] += 1
+    ms, _ = _time_launches(torch, step_narrow, max(steps, 6), warmup)
+    nbytes = nk * 2 + 4096 * 2 + 896 * 16 * 4
+    res["mmt4d_bf16_skinny_x86_tile_1x16x2_N14336_K4096"] = {
+        "kernel": lib.iree_uk_mi355x_last_kernel().decode(), "ms": round(ms, 5),
+        "value": round(nbytes / ms / 1e6, 1), "unit": "GB/s", "frac_of_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
     del rhs_set
 
     # The same with int4 weights (s8s4s32, tiles M0 x 16 x 32): N = 28672,
@@ -252,6 +269,28 @@ def _also(torch, lib, abi, synth, steps, warmup):
             entry["checksum_verified"] = bool(outs.to(torch.float64).sum().item() == want)
             del r, w, a
         res["mmt4d_s8s4s32_skinny_M%d_N28672_K8192" % m0] = entry
+    # The same 117 MB per copy read as int8 weights in the x86-64 VNNI matrix-vector tiles (s8s8s32 1x16x2):
+    # N = 28672, K = 4096. Checked through the sum of all outputs, as above.
+    lhs = torch.from_numpy(synth.uniform_int8(12, 30, 4096)).cuda()
+    outs = torch.zeros(n_i4, dtype=torch.int32, device="cuda")
+    ps = [_mmt4d_params(abi, lhs.data_ptr(), r.data_ptr(), outs.data_ptr(), 1, n_i4 // 16, 2048, 1, 16, 2,
+                        abi.MMT4D_TYPE_S8S8S32) for r in rhs_i4]
+    state = {"i": 0}
+
+    def step_vnni():
+        lib.iree_uk_mmt4d_p(C.byref(ps[state["i"] % 3]))
+        state["i"] += 1
+    ms, _ = _time_launches(torch, step_vnni, max(steps, 6), warmup)
+    nbytes = n_i4 * 4096 + 4096 + n_i4 * 4
+    entry = {"kernel": lib.iree_uk_mi355x_last_kernel().decode(), "ms": round(ms, 5),
+             "value": round(nbytes / ms / 1e6, 1), "unit": "GB/s", "frac_of_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+    lib.iree_uk_mmt4d_p(C.byref(ps[0]))
+    torch.cuda.synchronize()
+    w = rhs_i4[0].view(n_i4 // 16, 2048, 16, 2).to(torch.float64)
+    want = (lhs.view(2048, 2).to(torch.float64) * w.sum(dim=(0, 2))).sum().item()
+    entry["checksum_verified"] = bool(outs.to(torch.float64).sum().item() == want)
+    del w
+    res["mmt4d_s8s8s32_skinny_x86_tile_1x16x2_N28672_K4096"] = entry
     del rhs_i4
 
     # pack / unpack f32 [8191, 8190] <-> [512, 8190, 16, 1]; two buffer sets rotated

@@ -1,0 +1,298 @@
+// mmt4d for skinny left-hand sides in the narrow tile shapes that the
+// reference's CPU targets pick for them: at most 8 lhs rows in total (e.g.
+// M0 = 1, 2, 4 with M = 1) and row pieces (K0 elements) of 2, 4 or 8 bytes:
+// the x86-64 1x16x2 int8 / bf16 and 1x16x1 f16 / f32 tiles, the Arm 1x8x4 and
+// 1x8x8 int8 tiles and their 2- and 4-row siblings (mmt4d_x86_64_tiles.inl,
+// mmt4d_arm_64_tiles.inl). An HBM-bandwidth kernel.
+//
+// With pieces that short, 16 contiguous bytes of the rhs are several rows of
+// one k step, not one row: the wrong way round for an MFMA operand, and the
+// matrix kernels cannot load an lhs whose tiles are narrower than 16 bytes per
+// k step at all. Here nothing is transposed. The rhs of one tile row
+// (N0 rows x K k steps, one contiguous stream) is read 16 bytes per lane, and
+// each lane multiplies the 16 / G rows it holds with the lhs pieces of its
+// k step on the VALU (v_dot4_i32_i8, v_dot2_f32_f16, FMAs), keeping one
+// accumulator per (lhs row, rhs row). The lhs is small and comes through the
+// caches. At the end the lanes that hold the same rhs rows (they differ in
+// k step) are summed with a butterfly of lane exchanges, the wavefronts of the
+// workgroup (which split the stream between them) through LDS, both in a
+// fixed order, so results do not depend on scheduling.
+#include "uk_internal.h"
+
+namespace uk {
+namespace {
+
+typedef int v4i32 __attribute__((ext_vector_type(4)));
+typedef _Float16 v2f16 __attribute__((ext_vector_type(2)));
+
+enum Kind { kI8 = 0, kF16 = 1, kBF16 = 2, kF32 = 3 };
+
+struct SkinnyArgs {
+  const uint8_t* lhs;
+  const uint8_t* rhs;
+  uint8_t* out;
+  int64_t lhs_stride_bytes, rhs_stride_bytes;
+  int64_t out_stride0;  // elements
+  int64_t tile_bytes;   // K * N0 * G: one rhs tile row
+  int32_t rows;         // M * M0
+  int32_t N, K;
+  int32_t log2_M0, log2_N0;
+  int32_t accumulate;
+};
+
+template <int KIND> struct Acc { typedef float type; };
+template <> struct Acc<kI8> { typedef int32_t type; };
+
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
+__device__ __forceinline__ float f16_lo(uint32_t w) { return (float)__builtin_bit_cast(v2f16, w)[0]; }
+__device__ __forceinline__ float f16_hi(uint32_t w) { return (float)__builtin_bit_cast(v2f16, w)[1]; }
+
+// The lhs piece (G bytes) of one k step, zero-extended into two dwords.
+template <int G>
+__device__ __forceinline__ uint2 load_lhs_piece(const uint8_t* p) {
+  if constexpr (G == 2) return make_uint2(*(const uint16_t*)p, 0);
+  else if constexpr (G == 4) return make_uint2(*(const uint32_t*)p, 0);
+  else return *(const uint2*)p;
+}
+
+// acc[r] += (row r of the 16 / G rows in `v`) . (lhs piece l), all of one k step.
+template <int KIND, int G>
+__device__ __forceinline__ void multiply_piece(const uint4 v, const uint2 l, typename Acc<KIND>::type* acc) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+  if constexpr (KIND == kI8) {
+    if constexpr (G == 2) {
+      // Two rows per dword: the lhs pair in the low resp. high half, zeros in the other.
+      const int lo = (int)l.x, hi = (int)(l.x << 16);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc[2 * i] = __builtin_amdgcn_sdot4((int)w[i], lo, acc[2 * i], false);
+        acc[2 * i + 1] = __builtin_amdgcn_sdot4((int)w[i], hi, acc[2 * i + 1], false);
+      }
+    } else if constexpr (G == 4) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_sdot4((int)w[i], (int)l.x, acc[i], false);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        acc[i] = __builtin_amdgcn_sdot4((int)w[2 * i], (int)l.x, acc[i], false);
+        acc[i] = __builtin_amdgcn_sdot4((int)w[2 * i + 1], (int)l.y, acc[i], false);
+      }
+    }
+  } else if constexpr (KIND == kF32) {
+    if constexpr (G == 4) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] = fmaf(__uint_as_float(w[i]), __uint_as_float(l.x), acc[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        acc[i] = fmaf(__uint_as_float(w[2 * i]), __uint_as_float(l.x), acc[i]);
+        acc[i] = fmaf(__uint_as_float(w[2 * i + 1]), __uint_as_float(l.y), acc[i]);
+      }
+    }
+  } else {
+    // 16-bit floats, widened to f32 (exact) and accumulated in f32 in k0 order.
+    auto lo = [](uint32_t x) { return KIND == kF16 ? f16_lo(x) : bf16_lo(x); };
+    auto hi = [](uint32_t x) { return KIND == kF16 ? f16_hi(x) : bf16_hi(x); };
+    if constexpr (G == 2) {
+      const float l0 = lo(l.x);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc[2 * i] = fmaf(lo(w[i]), l0, acc[2 * i]);
+        acc[2 * i + 1] = fmaf(hi(w[i]), l0, acc[2 * i + 1]);
+      }
+    } else if constexpr (G == 4) {
+      const float l0 = lo(l.x), l1 = hi(l.x);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] = fmaf(hi(w[i]), l1, fmaf(lo(w[i]), l0, acc[i]));
+    } else {
+      const float l0 = lo(l.x), l1 = hi(l.x), l2 = lo(l.y), l3 = hi(l.y);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        acc[i] = fmaf(hi(w[2 * i]), l1, fmaf(lo(w[2 * i]), l0, acc[i]));
+        acc[i] = fmaf(hi(w[2 * i + 1]), l3, fmaf(lo(w[2 * i + 1]), l2, acc[i]));
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ int32_t exchange(int32_t v, int lane_xor) { return __shfl_xor(v, lane_xor, 64); }
+__device__ __forceinline__ float exchange(float v, int lane_xor) { return __shfl_xor(v, lane_xor, 64); }
+
+// G: bytes of a row piece; ROWS: lhs rows the kernel keeps accumulators for
+// (a.rows <= ROWS); UNROLL: 1 KiB blocks of the rhs stream a wavefront has in
+// flight. One workgroup of four wavefronts per rhs tile row.
+template <int KIND, int G, int ROWS, int UNROLL>
+__global__ __launch_bounds__(256) void mmt4d_skinny_kernel(const SkinnyArgs a) {
+  typedef typename Acc<KIND>::type acc_t;
+  constexpr int R = 16 / G;  // rhs rows in a lane's 16 bytes
+  __shared__ acc_t partial[4][ROWS][16];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int32_t M0 = 1 << a.log2_M0, N0 = 1 << a.log2_N0;
+  // One k step of the rhs is N0 * G bytes = `lanes_per_kstep` lanes; a block of
+  // 1 KiB holds whole k steps, so a lane keeps its rows from block to block.
+  const int log2_kstep_bytes = a.log2_N0 + (G == 2 ? 1 : (G == 4 ? 2 : 3));
+  const int log2_lanes_per_kstep = log2_kstep_bytes - 4;
+  const int32_t kstep_in_block = lane >> log2_lanes_per_kstep;
+  const int32_t lhs_kstep_bytes = G << a.log2_M0;
+
+  const uint8_t* rhs_tile = a.rhs + (int64_t)blockIdx.x * a.rhs_stride_bytes;
+  const uint8_t* lhs_row[ROWS];
+#pragma unroll
+  for (int m = 0; m < ROWS; ++m) {
+    const int row = m < a.rows ? m : a.rows - 1;  // clamp: computed, not stored
+    lhs_row[m] = a.lhs + (int64_t)(row >> a.log2_M0) * a.lhs_stride_bytes + (row & (M0 - 1)) * G;
+  }
+
+  acc_t acc[ROWS][R];
+#pragma unroll
+  for (int m = 0; m < ROWS; ++m)
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[m][r] = 0;
+
+  const int64_t blocks = (a.tile_bytes + 1023) >> 10;
+  for (int64_t j0 = wave; j0 < blocks; j0 += 4 * UNROLL) {
+    uint4 v[UNROLL];
+    uint2 l[UNROLL][ROWS];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int64_t off = ((j0 + 4 * u) << 10) + 16 * lane;
+      const bool inside = off < a.tile_bytes;
+      v[u] = make_uint4(0, 0, 0, 0);
+      if (inside) v[u] = __builtin_bit_cast(uint4, __builtin_nontemporal_load((const v4i32*)(rhs_tile + off)));
+      // The lhs piece of this lane's k step.
+      const int64_t kstep = inside ? ((j0 + 4 * u) << (10 - log2_kstep_bytes)) + kstep_in_block : 0;
+#pragma unroll
+      for (int m = 0; m < ROWS; ++m) {
+        l[u][m] = load_lhs_piece<G>(lhs_row[m] + kstep * lhs_kstep_bytes);
+        if (!inside) l[u][m] = make_uint2(0, 0);  // 0 * 0, whatever the lhs holds there
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+      for (int m = 0; m < ROWS; ++m) multiply_piece<KIND, G>(v[u], l[u][m], acc[m]);
+  }
+
+  // Lanes that are a multiple of lanes_per_kstep apart hold the same rhs rows.
+  for (int s = 1 << log2_lanes_per_kstep; s < 64; s <<= 1) {
+#pragma unroll
+    for (int m = 0; m < ROWS; ++m)
+#pragma unroll
+      for (int r = 0; r < R; ++r) acc[m][r] += exchange(acc[m][r], s);
+  }
+  if (lane < (1 << log2_lanes_per_kstep)) {
+#pragma unroll
+    for (int m = 0; m < ROWS; ++m)
+#pragma unroll
+      for (int r = 0; r < R; ++r) partial[wave][m][R * lane + r] = acc[m][r];
+  }
+  __syncthreads();
+  const int t = threadIdx.x;
+  const int m = t >> a.log2_N0, j0 = t & (N0 - 1);
+  if (m < a.rows) {
+    acc_t sum = partial[0][m][j0];
+    sum += partial[1][m][j0];
+    sum += partial[2][m][j0];
+    sum += partial[3][m][j0];
+    acc_t* dst = (acc_t*)a.out + (int64_t)(m >> a.log2_M0) * a.out_stride0 +
+                 ((int64_t)blockIdx.x << (a.log2_M0 + a.log2_N0)) + ((m & (M0 - 1)) << a.log2_N0) + j0;
+    if (a.accumulate) sum += *dst;
+    *dst = sum;
+  }
+}
+
+int log2_exact(int64_t v) {
+  if (v <= 0 || (v & (v - 1))) return -1;
+  int l = 0;
+  while ((1ll << l) < v) ++l;
+  return l;
+}
+
+bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, int* piece_bytes, SkinnyArgs* s) {
+  int elem_bytes;
+  switch (a.flags & IREE_UK_FLAG_MMT4D_TYPE_MASK) {
+    case IREE_UK_FLAG_MMT4D_TYPE_S8S8S32: *kind = kI8; elem_bytes = 1; break;
+    case IREE_UK_FLAG_MMT4D_TYPE_F16F16F32: *kind = kF16; elem_bytes = 2; break;
+    case IREE_UK_FLAG_MMT4D_TYPE_BF16BF16F32: *kind = kBF16; elem_bytes = 2; break;
+    case IREE_UK_FLAG_MMT4D_TYPE_F32F32F32: *kind = kF32; elem_bytes = 4; break;
+    default: return false;
+  }
+  const int g = a.K0 * elem_bytes;
+  if (g != 2 && g != 4 && g != 8) return false;
+  const int lm0 = log2_exact(a.M0), ln0 = log2_exact(a.N0);
+  // A k step of the rhs must be whole 16-byte vectors.
+  if (lm0 < 0 || ln0 < 0 || a.M0 > 8 || a.N0 > 16 || a.N0 * g < 16) return false;
+  *piece_bytes = g;
+  if (probe_only) return a.M0 * g < 16;  // what no matrix kernel takes
+  if (a.M * a.M0 > 8 || a.M <= 0 || a.K <= 0 || a.N <= 0 || a.N > 0x7FFFFFFF) return false;
+  const int64_t lhs_stride_bytes = a.lhs_stride0 * elem_bytes, rhs_stride_bytes = a.rhs_stride0 * elem_bytes;
+  if ((uintptr_t)a.rhs % 16 || (a.N > 1 && rhs_stride_bytes % 16)) return false;
+  if ((uintptr_t)a.lhs % g || (a.M > 1 && lhs_stride_bytes % g)) return false;
+  if ((uintptr_t)a.out % 4) return false;
+  s->lhs = a.lhs; s->rhs = a.rhs; s->out = a.out;
+  s->lhs_stride_bytes = lhs_stride_bytes;
+  s->rhs_stride_bytes = rhs_stride_bytes;
+  s->out_stride0 = a.out_stride0;
+  s->tile_bytes = a.K * a.N0 * g;
+  s->rows = (int32_t)(a.M * a.M0);
+  s->N = (int32_t)a.N;
+  s->K = (int32_t)a.K;
+  s->log2_M0 = lm0;
+  s->log2_N0 = ln0;
+  s->accumulate = (a.flags & IREE_UK_FLAG_MMT4D_ACCUMULATE) ? 1 : 0;
+  return true;
+}
+
+template <int KIND, int G>
+hipError_t launch_piece(const SkinnyArgs& s, hipStream_t stream) {
+  // Fewer lhs rows leave registers for more of the rhs stream in flight.
+  const dim3 grid((unsigned)s.N), block(256);
+  if (s.rows <= 1) hipLaunchKernelGGL((mmt4d_skinny_kernel<KIND, G, 1, 16>), grid, block, 0, stream, s);
+  else if (s.rows <= 2) hipLaunchKernelGGL((mmt4d_skinny_kernel<KIND, G, 2, 16>), grid, block, 0, stream, s);
+  else if (s.rows <= 4) hipLaunchKernelGGL((mmt4d_skinny_kernel<KIND, G, 4, 8>), grid, block, 0, stream, s);
+  else hipLaunchKernelGGL((mmt4d_skinny_kernel<KIND, G, 8, 4>), grid, block, 0, stream, s);
+  return hipGetLastError();
+}
+
+template <int KIND>
+hipError_t launch_kind(const SkinnyArgs& s, int piece_bytes, hipStream_t stream) {
+  if (piece_bytes == 4) return launch_piece<KIND, 4>(s, stream);
+  if (piece_bytes == 8) return launch_piece<KIND, 8>(s, stream);
+  if constexpr (KIND != kF32) return launch_piece<KIND, 2>(s, stream);
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_skinny(const Mmt4dArgs& a, hipStream_t stream, const char** name) {
+  int kind, piece_bytes;
+  SkinnyArgs s;
+  if (!make_args(a, false, &kind, &piece_bytes, &s)) return hipErrorInvalidValue;
+  *name = "mmt4d_skinny";
+  switch (kind) {
+    case kI8: return launch_kind<kI8>(s, piece_bytes, stream);
+    case kF16: return launch_kind<kF16>(s, piece_bytes, stream);
+    case kBF16: return launch_kind<kBF16>(s, piece_bytes, stream);
+    default: return launch_kind<kF32>(s, piece_bytes, stream);
+  }
+}
+
+}  // namespace
+
+// Measured on 1 x 14336 x 4096 problems: with up to 4 lhs rows this kernel is
+// at the HBM rate (bf16 1x16x2 18 us, int8 1x16x2 10 us) and level with the
+// 64x64 matrix kernel where that applies; with 8 rows it is VALU bound (int8
+// 8x16x2 41 us against 23 us, bf16 8x16x2 32 against 23 us).
+bool mmt4d_skinny_preferred(const Mmt4dArgs& a) {
+  int lhs_bits, rhs_bits, out_bits;
+  if (!mmt4d_type_bits(a.flags, &lhs_bits, &rhs_bits, &out_bits)) return false;
+  return a.M * a.M0 <= 4 || a.M0 * a.K0 * lhs_bits / 8 < 16;
+}
+
+Mmt4dLauncher select_mmt4d_skinny(const Mmt4dArgs& a, bool probe_only) {
+  int kind, piece_bytes;
+  SkinnyArgs s;
+  return make_args(a, probe_only, &kind, &piece_bytes, &s) ? launch_skinny : nullptr;
+}
+
+}  // namespace uk

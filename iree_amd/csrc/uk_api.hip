@@ -161,8 +161,10 @@ bool launch_ok(hipError_t e, const char* what) {
 uk::Mmt4dLauncher select_mmt4d(const uk::Mmt4dArgs& a, bool probe_only) {
   uk::Mmt4dLauncher l = nullptr;
   if ((l = uk::select_mmt4d_gemv(a, probe_only))) return l;
+  const uk::Mmt4dLauncher skinny = uk::select_mmt4d_skinny(a, probe_only);
+  if (skinny && (probe_only || uk::mmt4d_skinny_preferred(a))) return skinny;
   if ((l = uk::select_mmt4d_mfma(a, probe_only))) return l;
-  return nullptr;
+  return skinny;
 }
 
 int pack_elem_bytes(uint32_t flags) {

@@ -57,6 +57,9 @@ typedef hipError_t (*Mmt4dLauncher)(const Mmt4dArgs& a, hipStream_t stream, cons
 // problems carry only type flags and M0/N0/K0 (used by iree_uk_mmt4d_info).
 Mmt4dLauncher select_mmt4d_mfma(const Mmt4dArgs& a, bool probe_only);
 Mmt4dLauncher select_mmt4d_gemv(const Mmt4dArgs& a, bool probe_only);
+Mmt4dLauncher select_mmt4d_skinny(const Mmt4dArgs& a, bool probe_only);
+// Whether the skinny kernel beats a matrix kernel that also covers the problem.
+bool mmt4d_skinny_preferred(const Mmt4dArgs& a);
 
 // The in-dispatch int8 microkernel over a grid of data-tiled tiles (multi_mma.hip).
 hipError_t launch_multi_mma_i8(const void* a, const void* b, void* c, int64_t outer_m, int64_t outer_n, int32_t k_size,

@@ -1,0 +1,76 @@
+"""GPU parity for the skinny-lhs kernel of the narrow tile shapes (mmt4d_skinny.hip): at most 8 lhs rows in total
+and row pieces (K0 elements) of 2, 4 or 8 bytes, i.e. what the reference's CPU targets pick for matrix-vector and
+few-row products (mmt4d_x86_64_tiles.inl: 1x16x2 int8/bf16, 1x16x1 f16/f32 and their 2-, 4- and 8-row siblings;
+mmt4d_arm_64_tiles.inl: 1x8x4 and 1x8x8 int8, 1x8x1 f32, ...).
+
+Integer results are compared bit for bit with a float64 matrix product of the same operands, float results within
+|got - ref| <= 1e-3 * max(|ref|, rms(ref)) of it (test_gpu_big_tiles.run_case).
+"""
+import ctypes as C
+
+import pytest
+import torch
+
+from iree_amd import abi
+from test_gpu_big_tiles import run_case
+from test_gpu_configs import gpu_lib, mm_params  # noqa: F401
+
+pytestmark = pytest.mark.gpu
+
+S8, F16, BF16, F32 = abi.MMT4D_TYPE_S8S8S32, abi.MMT4D_TYPE_F16F16F32, abi.MMT4D_TYPE_BF16BF16F32, abi.MMT4D_TYPE_F32F32F32
+
+
+# (type, M, M0, N0, K0): every piece size of every type, every row count, both rhs tile heights, several lhs tiles.
+SHAPES = [
+    (S8, 1, 1, 16, 2), (S8, 1, 2, 16, 2), (S8, 1, 4, 16, 2), (S8, 2, 4, 16, 2), (S8, 3, 1, 16, 2), (S8, 2, 2, 8, 2),
+    (S8, 1, 1, 8, 4), (S8, 1, 2, 8, 4), (S8, 1, 4, 16, 4), (S8, 5, 1, 4, 4), (S8, 1, 1, 8, 8), (S8, 1, 4, 8, 8),
+    (S8, 2, 4, 2, 8), (F16, 1, 1, 16, 1), (F16, 1, 4, 16, 1), (F16, 7, 1, 8, 1), (F16, 1, 2, 8, 2), (F16, 1, 1, 16, 4),
+    (BF16, 1, 1, 16, 2), (BF16, 1, 2, 16, 2), (BF16, 8, 1, 16, 1), (BF16, 3, 1, 8, 4), (F32, 1, 1, 16, 1),
+    (F32, 1, 4, 8, 1), (F32, 2, 2, 4, 1), (F32, 1, 1, 8, 2), (F32, 6, 1, 2, 2)]
+
+
+@pytest.mark.parametrize("flags,M,M0,N0,K0", SHAPES)
+def test_narrow_tiles_few_rows(gpu_lib, flags, M, M0, N0, K0):
+    # K: less than one 1 KiB block of the stream, a stream that ends inside a block and inside a wavefront's share,
+    # and one long enough for several rounds of every wavefront.
+    for n, K in enumerate((3, 77, 1500)):
+        run_case(gpu_lib, flags, M, 37 + n, K, M0, N0, K0, "mmt4d_skinny", accumulate=bool(n & 1), seed=K + M0)
+    # strided operands with offsets (rhs tile rows stay 16-byte aligned, lhs rows 8-byte), padded output
+    e = 1 if flags == S8 else (4 if flags == F32 else 2)
+    run_case(gpu_lib, flags, M, 21, 130, M0, N0, K0, "mmt4d_skinny", lhs_pad=8, rhs_pad=16 // e, out_pad=5,
+             offsets=(8, 32 // e, 3), accumulate=True, seed=9)
+
+
+def test_non_finite_lhs_values_do_not_leak_into_other_k_steps(gpu_lib):
+    # The rhs stream of a tile row ends inside a block of 64 lanes x 16 bytes; the idle lanes must add nothing, also
+    # when the lhs holds an infinity at the k step they would read.
+    M0, N0, K0, K, N = 1, 16, 2, 5, 3
+    lhs = torch.ones(K * M0 * K0, device="cuda", dtype=torch.bfloat16)
+    lhs[0] = float("inf")
+    rhs = torch.ones(N * K * N0 * K0, device="cuda", dtype=torch.bfloat16)
+    rhs.view(N, K, N0, K0)[:, 0, :, 0] = 0.25
+    rhs.view(N, K, N0, K0)[:, 0, 5, 0] = 0.0  # inf * 0 = nan in exactly these outputs
+    out = torch.zeros(N * M0 * N0, device="cuda")
+    p = mm_params(lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), 1, N, K, M0, N0, K0, BF16)
+    gpu_lib.iree_uk_mmt4d_p(C.byref(p))
+    assert gpu_lib.iree_uk_mi355x_last_kernel() == b"mmt4d_skinny"
+    got = out.view(N, N0)
+    assert bool(torch.isnan(got[:, 5]).all())
+    rest = torch.cat([got[:, :5], got[:, 6:]], dim=1)
+    assert bool(torch.isinf(rest).all()) and bool((rest > 0).all())
+
+
+def test_eight_row_tiles_a_matrix_kernel_can_load_go_there(gpu_lib):
+    # More than 4 rows make this kernel VALU bound; 8x16x2 int8 tiles are 16 bytes per k step, which the matrix
+    # kernels load directly.
+    run_case(gpu_lib, S8, 1, 40, 64, 8, 16, 2, "mmt4d_mfma_64x64", accumulate=True)
+    run_case(gpu_lib, BF16, 1, 40, 64, 8, 16, 1, "mmt4d_mfma_64x64")
+    # ... unless it cannot (lhs rows only 8-byte aligned)
+    run_case(gpu_lib, S8, 1, 40, 64, 8, 16, 2, "mmt4d_skinny", offsets=(8, 0, 0))
+
+
+def test_more_rows_than_the_kernel_takes_fall_through(gpu_lib):
+    # 9 rows of 1x16x2 int8 tiles: no matrix kernel loads such an lhs either; the generic kernel, still exact.
+    run_case(gpu_lib, S8, 9, 20, 40, 1, 16, 2, "mmt4d_generic", accumulate=True)
+    # rhs tile rows that are not 16-byte aligned
+    run_case(gpu_lib, S8, 1, 20, 40, 1, 16, 2, "mmt4d_generic", rhs_pad=2)
