@@ -59,7 +59,7 @@ bool make_plan(const Mmt4dArgs& a, bool probe_only, Plan* plan) {
     gather = 16;
   } else if (lhs_rb >= 16 && lhs_rb <= 64) {
     gather = 16;
-  } else if (lhs_rb == 4 || ((lhs_rb == 2 || lhs_rb == 8) && !narrow)) {
+  } else if (lhs_rb == 4 || lhs_rb == 2 || lhs_rb == 8) {
     // 2 and 8 (e.g. the x86-64 int8 16x16x2 and f16 16x16x1 tiles, the Arm int8
     // 8x8x8 tiles) run on the direct-to-LDS kernel only: see below.
     gather = lhs_rb;
@@ -79,7 +79,8 @@ bool make_plan(const Mmt4dArgs& a, bool probe_only, Plan* plan) {
   const int64_t rhs_stride_bytes = i4 ? a.rhs_stride0 / 2 : a.rhs_stride0 * elem_bytes;
   if (((uintptr_t)a.lhs % lhs_align) || (a.M > 1 && lhs_stride_bytes % lhs_align)) return false;
   if (((uintptr_t)a.rhs % rhs_align) || (a.N > 1 && rhs_stride_bytes % rhs_align)) return false;
-  if (((uintptr_t)a.out % 16) || (a.M > 1 && a.out_stride0 % 4)) return false;
+  // (four consecutive outputs per store: 16 bytes, 8 with a 16-bit output)
+  if (((uintptr_t)a.out % (narrow ? 8 : 16)) || (a.M > 1 && a.out_stride0 % 4)) return false;
   // Per-piece offsets from a workgroup's first tile are kept in 32 bits.
   const int64_t lhs_reach = ((256 >> lm0) + 1) * lhs_stride_bytes + 80 * ((int64_t)lhs_rb << lm0);
   const int64_t rhs_reach = ((256 >> ln0) + 1) * rhs_stride_bytes + 80 * ((int64_t)rhs_rb << ln0);

@@ -6,9 +6,7 @@
 namespace uk {
 
 hipError_t launch_mfma_f16(const MfmaArgs& m, int gather, bool narrow, hipStream_t stream, const char** name) {
-  if (narrow)
-    return gather == 16 ? launch_variant<kF16, false, 16, true>(m, stream, name)
-                        : launch_variant<kF16, false, 4, true>(m, stream, name);
+  if (narrow) return launch_mfma_f16_narrow(m, gather, stream, name);
   switch (gather) {
     case 16: return launch_variant<kF16, false, 16, false>(m, stream, name);
     case 8: return launch_variant<kF16, false, 8, false>(m, stream, name);

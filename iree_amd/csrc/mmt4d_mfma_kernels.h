@@ -74,6 +74,8 @@ hipError_t launch_mfma_i8(const MfmaArgs& m, int gather, bool rhs_i4, hipStream_
 hipError_t launch_mfma_f16(const MfmaArgs& m, int gather, bool narrow, hipStream_t stream, const char** name);
 hipError_t launch_mfma_bf16(const MfmaArgs& m, int gather, bool narrow, hipStream_t stream, const char** name);
 hipError_t launch_mfma_f32(const MfmaArgs& m, int gather, hipStream_t stream, const char** name);
+hipError_t launch_mfma_f16_narrow(const MfmaArgs& m, int gather, hipStream_t stream, const char** name);
+hipError_t launch_mfma_bf16_narrow(const MfmaArgs& m, int gather, hipStream_t stream, const char** name);
 
 // Whether the direct-to-LDS kernel covers the problem with row pieces of
 // `gather` bytes (2 and 8 have no other MFMA kernel).

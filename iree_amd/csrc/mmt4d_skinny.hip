@@ -17,6 +17,11 @@
 // k step) are summed with a butterfly of lane exchanges, the wavefronts of the
 // workgroup (which split the stream between them) through LDS, both in a
 // fixed order, so results do not depend on scheduling.
+//
+// f16f16f16 and bf16bf16bf16 are taken with the flag that skips the roundings
+// between k steps (mmt4d_tile_generic.c:229-286, 319-376): f32 accumulators,
+// one rounding to the 16-bit output at the end.
+#include "uk_device.h"
 #include "uk_internal.h"
 
 namespace uk {
@@ -121,9 +126,11 @@ __device__ __forceinline__ float exchange(float v, int lane_xor) { return __shfl
 
 // G: bytes of a row piece; ROWS: lhs rows the kernel keeps accumulators for
 // (a.rows <= ROWS); UNROLL: 1 KiB blocks of the rhs stream a wavefront has in
-// flight. One workgroup of four wavefronts per rhs tile row.
-template <int KIND, int G, int ROWS, int UNROLL>
+// flight; NARROW: the output has the 16-bit type of the operands. One
+// workgroup of four wavefronts per rhs tile row.
+template <int KIND, int G, int ROWS, int UNROLL, bool NARROW>
 __global__ __launch_bounds__(256) void mmt4d_skinny_kernel(const SkinnyArgs a) {
+  static_assert(!NARROW || KIND == kF16 || KIND == kBF16, "16-bit outputs are floats");
   typedef typename Acc<KIND>::type acc_t;
   constexpr int R = 16 / G;  // rhs rows in a lane's 16 bytes
   __shared__ acc_t partial[4][ROWS][16];
@@ -196,10 +203,18 @@ __global__ __launch_bounds__(256) void mmt4d_skinny_kernel(const SkinnyArgs a) {
     sum += partial[1][m][j0];
     sum += partial[2][m][j0];
     sum += partial[3][m][j0];
-    acc_t* dst = (acc_t*)a.out + (int64_t)(m >> a.log2_M0) * a.out_stride0 +
-                 ((int64_t)blockIdx.x << (a.log2_M0 + a.log2_N0)) + ((m & (M0 - 1)) << a.log2_N0) + j0;
-    if (a.accumulate) sum += *dst;
-    *dst = sum;
+    const int64_t index = (int64_t)(m >> a.log2_M0) * a.out_stride0 +
+                          ((int64_t)blockIdx.x << (a.log2_M0 + a.log2_N0)) + ((m & (M0 - 1)) << a.log2_N0) + j0;
+    if constexpr (NARROW) {
+      constexpr int EBITS = KIND == kF16 ? 5 : 8;
+      uint16_t* dst = (uint16_t*)a.out + index;
+      if (a.accumulate) sum += widen16<EBITS>(*dst);
+      *dst = narrow16<EBITS>(sum);
+    } else {
+      acc_t* dst = (acc_t*)a.out + index;
+      if (a.accumulate) sum += *dst;
+      *dst = sum;
+    }
   }
 }
 
@@ -210,13 +225,23 @@ int log2_exact(int64_t v) {
   return l;
 }
 
-bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, int* piece_bytes, SkinnyArgs* s) {
+bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, int* piece_bytes, bool* narrow, SkinnyArgs* s) {
   int elem_bytes;
+  *narrow = false;
+  const bool skip_roundings = a.flags & IREE_UK_FLAG_MMT4D_SKIP_INTERMEDIATE_ROUNDINGS;
   switch (a.flags & IREE_UK_FLAG_MMT4D_TYPE_MASK) {
     case IREE_UK_FLAG_MMT4D_TYPE_S8S8S32: *kind = kI8; elem_bytes = 1; break;
     case IREE_UK_FLAG_MMT4D_TYPE_F16F16F32: *kind = kF16; elem_bytes = 2; break;
     case IREE_UK_FLAG_MMT4D_TYPE_BF16BF16F32: *kind = kBF16; elem_bytes = 2; break;
     case IREE_UK_FLAG_MMT4D_TYPE_F32F32F32: *kind = kF32; elem_bytes = 4; break;
+    case IREE_UK_FLAG_MMT4D_TYPE_F16F16F16:
+      if (!skip_roundings) return false;
+      *kind = kF16; elem_bytes = 2; *narrow = true;
+      break;
+    case IREE_UK_FLAG_MMT4D_TYPE_BF16BF16BF16:
+      if (!skip_roundings) return false;
+      *kind = kBF16; elem_bytes = 2; *narrow = true;
+      break;
     default: return false;
   }
   const int g = a.K0 * elem_bytes;
@@ -230,7 +255,7 @@ bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, int* piece_bytes,
   const int64_t lhs_stride_bytes = a.lhs_stride0 * elem_bytes, rhs_stride_bytes = a.rhs_stride0 * elem_bytes;
   if ((uintptr_t)a.rhs % 16 || (a.N > 1 && rhs_stride_bytes % 16)) return false;
   if ((uintptr_t)a.lhs % g || (a.M > 1 && lhs_stride_bytes % g)) return false;
-  if ((uintptr_t)a.out % 4) return false;
+  if ((uintptr_t)a.out % (*narrow ? 2 : 4)) return false;
   s->lhs = a.lhs; s->rhs = a.rhs; s->out = a.out;
   s->lhs_stride_bytes = lhs_stride_bytes;
   s->rhs_stride_bytes = rhs_stride_bytes;
@@ -245,35 +270,38 @@ bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, int* piece_bytes,
   return true;
 }
 
-template <int KIND, int G>
+template <int KIND, int G, bool NARROW>
 hipError_t launch_piece(const SkinnyArgs& s, hipStream_t stream) {
   // Fewer lhs rows leave registers for more of the rhs stream in flight.
   const dim3 grid((unsigned)s.N), block(256);
-  if (s.rows <= 1) hipLaunchKernelGGL((mmt4d_skinny_kernel<KIND, G, 1, 16>), grid, block, 0, stream, s);
-  else if (s.rows <= 2) hipLaunchKernelGGL((mmt4d_skinny_kernel<KIND, G, 2, 16>), grid, block, 0, stream, s);
-  else if (s.rows <= 4) hipLaunchKernelGGL((mmt4d_skinny_kernel<KIND, G, 4, 8>), grid, block, 0, stream, s);
-  else hipLaunchKernelGGL((mmt4d_skinny_kernel<KIND, G, 8, 4>), grid, block, 0, stream, s);
+  if (s.rows <= 1) hipLaunchKernelGGL((mmt4d_skinny_kernel<KIND, G, 1, 16, NARROW>), grid, block, 0, stream, s);
+  else if (s.rows <= 2) hipLaunchKernelGGL((mmt4d_skinny_kernel<KIND, G, 2, 16, NARROW>), grid, block, 0, stream, s);
+  else if (s.rows <= 4) hipLaunchKernelGGL((mmt4d_skinny_kernel<KIND, G, 4, 8, NARROW>), grid, block, 0, stream, s);
+  else hipLaunchKernelGGL((mmt4d_skinny_kernel<KIND, G, 8, 4, NARROW>), grid, block, 0, stream, s);
   return hipGetLastError();
 }
 
-template <int KIND>
+template <int KIND, bool NARROW>
 hipError_t launch_kind(const SkinnyArgs& s, int piece_bytes, hipStream_t stream) {
-  if (piece_bytes == 4) return launch_piece<KIND, 4>(s, stream);
-  if (piece_bytes == 8) return launch_piece<KIND, 8>(s, stream);
-  if constexpr (KIND != kF32) return launch_piece<KIND, 2>(s, stream);
+  if (piece_bytes == 4) return launch_piece<KIND, 4, NARROW>(s, stream);
+  if (piece_bytes == 8) return launch_piece<KIND, 8, NARROW>(s, stream);
+  if constexpr (KIND != kF32) return launch_piece<KIND, 2, NARROW>(s, stream);
   return hipErrorInvalidValue;
 }
 
 hipError_t launch_skinny(const Mmt4dArgs& a, hipStream_t stream, const char** name) {
   int kind, piece_bytes;
+  bool narrow;
   SkinnyArgs s;
-  if (!make_args(a, false, &kind, &piece_bytes, &s)) return hipErrorInvalidValue;
+  if (!make_args(a, false, &kind, &piece_bytes, &narrow, &s)) return hipErrorInvalidValue;
   *name = "mmt4d_skinny";
   switch (kind) {
-    case kI8: return launch_kind<kI8>(s, piece_bytes, stream);
-    case kF16: return launch_kind<kF16>(s, piece_bytes, stream);
-    case kBF16: return launch_kind<kBF16>(s, piece_bytes, stream);
-    default: return launch_kind<kF32>(s, piece_bytes, stream);
+    case kI8: return launch_kind<kI8, false>(s, piece_bytes, stream);
+    case kF16:
+      return narrow ? launch_kind<kF16, true>(s, piece_bytes, stream) : launch_kind<kF16, false>(s, piece_bytes, stream);
+    case kBF16:
+      return narrow ? launch_kind<kBF16, true>(s, piece_bytes, stream) : launch_kind<kBF16, false>(s, piece_bytes, stream);
+    default: return launch_kind<kF32, false>(s, piece_bytes, stream);
   }
 }
 
@@ -291,8 +319,9 @@ bool mmt4d_skinny_preferred(const Mmt4dArgs& a) {
 
 Mmt4dLauncher select_mmt4d_skinny(const Mmt4dArgs& a, bool probe_only) {
   int kind, piece_bytes;
+  bool narrow;
   SkinnyArgs s;
-  return make_args(a, probe_only, &kind, &piece_bytes, &s) ? launch_skinny : nullptr;
+  return make_args(a, probe_only, &kind, &piece_bytes, &narrow, &s) ? launch_skinny : nullptr;
 }
 
 }  // namespace uk

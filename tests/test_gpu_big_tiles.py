@@ -157,7 +157,8 @@ def test_oblong_tiles_ragged(gpu_lib, flags, M0, N0, K0, K):
 @pytest.mark.parametrize("flags,M0,N0,K0,K", [
     (abi.MMT4D_TYPE_S8S8S32, 16, 16, 2, 96), (abi.MMT4D_TYPE_S8S8S32, 8, 8, 2, 64), (abi.MMT4D_TYPE_S8S8S32, 8, 8, 8, 24),
     (abi.MMT4D_TYPE_S8S8S32, 2, 8, 8, 8), (abi.MMT4D_TYPE_F16F16F32, 16, 16, 1, 64), (abi.MMT4D_TYPE_F16F16F32, 8, 8, 4, 16),
-    (abi.MMT4D_TYPE_BF16BF16F32, 8, 8, 4, 24), (abi.MMT4D_TYPE_BF16BF16F32, 16, 8, 1, 96), (abi.MMT4D_TYPE_F32F32F32, 8, 8, 2, 24)])
+    (abi.MMT4D_TYPE_BF16BF16F32, 8, 8, 4, 24), (abi.MMT4D_TYPE_BF16BF16F32, 16, 8, 1, 96), (abi.MMT4D_TYPE_F32F32F32, 8, 8, 2, 24),
+    (abi.MMT4D_TYPE_BF16BF16BF16, 8, 8, 4, 24), (abi.MMT4D_TYPE_F16F16F16, 8, 8, 1, 32)])
 def test_narrow_and_8_byte_row_pieces(gpu_lib, flags, M0, N0, K0, K):
     # 256x256 blocks, ragged in both directions, accumulating, padded output rows
     M, N = 3608 // M0 + 1, 3704 // N0 + 1
@@ -171,7 +172,8 @@ def test_narrow_and_8_byte_row_pieces(gpu_lib, flags, M0, N0, K0, K):
 # fragments of an operand (rows 2r / 2r+1 of 64 from one dword), which the epilogue has to undo: every block tile, with
 # the lhs paired and the rhs not (128x64), ragged edges that cut pairs apart, accumulation and padded output rows.
 @pytest.mark.parametrize("flags,M0,N0,K0,K", [(abi.MMT4D_TYPE_S8S8S32, 16, 16, 2, 64), (abi.MMT4D_TYPE_S8S8S32, 8, 8, 2, 32),
-                                              (abi.MMT4D_TYPE_F16F16F32, 16, 16, 1, 96), (abi.MMT4D_TYPE_BF16BF16F32, 8, 16, 1, 32)])
+                                              (abi.MMT4D_TYPE_F16F16F32, 16, 16, 1, 96), (abi.MMT4D_TYPE_BF16BF16F32, 8, 16, 1, 32),
+                                              (abi.MMT4D_TYPE_F16F16F16, 16, 16, 1, 32), (abi.MMT4D_TYPE_BF16BF16BF16, 16, 8, 1, 64)])
 def test_two_byte_row_pieces_on_every_block_tile(gpu_lib, flags, M0, N0, K0, K):
     n_cols = 14300 // N0 * N0
     run_case(gpu_lib, flags, 504 // M0, n_cols // N0, K, M0, N0, K0, "mmt4d_mfma_256x128", accumulate=True, out_pad=8, seed=K)

@@ -18,6 +18,7 @@ from test_gpu_configs import gpu_lib, mm_params  # noqa: F401
 pytestmark = pytest.mark.gpu
 
 S8, F16, BF16, F32 = abi.MMT4D_TYPE_S8S8S32, abi.MMT4D_TYPE_F16F16F32, abi.MMT4D_TYPE_BF16BF16F32, abi.MMT4D_TYPE_F32F32F32
+F16_OUT16, BF16_OUT16 = abi.MMT4D_TYPE_F16F16F16, abi.MMT4D_TYPE_BF16BF16BF16  # run with the roundings between k steps skipped
 
 
 # (type, M, M0, N0, K0): every piece size of every type, every row count, both rhs tile heights, several lhs tiles.
@@ -26,7 +27,9 @@ SHAPES = [
     (S8, 1, 1, 8, 4), (S8, 1, 2, 8, 4), (S8, 1, 4, 16, 4), (S8, 5, 1, 4, 4), (S8, 1, 1, 8, 8), (S8, 1, 4, 8, 8),
     (S8, 2, 4, 2, 8), (F16, 1, 1, 16, 1), (F16, 1, 4, 16, 1), (F16, 7, 1, 8, 1), (F16, 1, 2, 8, 2), (F16, 1, 1, 16, 4),
     (BF16, 1, 1, 16, 2), (BF16, 1, 2, 16, 2), (BF16, 8, 1, 16, 1), (BF16, 3, 1, 8, 4), (F32, 1, 1, 16, 1),
-    (F32, 1, 4, 8, 1), (F32, 2, 2, 4, 1), (F32, 1, 1, 8, 2), (F32, 6, 1, 2, 2)]
+    (F32, 1, 4, 8, 1), (F32, 2, 2, 4, 1), (F32, 1, 1, 8, 2), (F32, 6, 1, 2, 2), (F16_OUT16, 1, 1, 16, 1),
+    (F16_OUT16, 1, 4, 8, 1), (F16_OUT16, 3, 2, 8, 2), (BF16_OUT16, 1, 1, 16, 2), (BF16_OUT16, 1, 2, 8, 4),
+    (BF16_OUT16, 5, 1, 8, 4)]
 
 
 @pytest.mark.parametrize("flags,M,M0,N0,K0", SHAPES)
