@@ -101,20 +101,22 @@ def test_pack_unpack_random_cases(gpu_lib, oracle_lib, seed, small_elements_tran
     assert small_elements_transposed or b"unpack_tiled" in kernels
 
 
-def test_mmt4d_random_cases(gpu_lib, oracle_lib):
-    rnd = random.Random(1)
-    types = [abi.MMT4D_TYPE_S8S8S32, abi.MMT4D_TYPE_S8S4S32, abi.MMT4D_TYPE_F16F16F32, abi.MMT4D_TYPE_BF16BF16F32]
+def _mmt4d_sweep(gpu_lib, oracle_lib, seed, cases, types, n0_choices, long_k):
+    """Random problems of the given type flags against the oracle; returns the kernels that ran."""
+    rnd = random.Random(seed)
     kernels = set()
-    for case in range(300):
+    for case in range(cases):
         typ = rnd.choice(types)
-        lb, rb, _ = abi.MMT4D_BITS[typ]
-        M0, N0 = rnd.choice([1, 2, 4, 8, 16]), rnd.choice([4, 8, 16, 16])
-        K0 = rnd.choice([1, 2, 4, 8, 16, 32, 64])
+        lb, rb, ob = abi.MMT4D_BITS[typ & abi.MMT4D_TYPE_MASK]
+        M0, N0 = rnd.choice([1, 2, 4, 8, 16]), rnd.choice(n0_choices)
+        K0 = rnd.choice([1, 2, 4, 8, 16, 32, 64] if lb < 32 else [1, 2, 4, 8, 16])
         if typ == abi.MMT4D_TYPE_S8S4S32 and K0 < 2:
             K0 = 2
         kind = rnd.random()
         if kind < 0.35:      # a skinny lhs against many rhs tiles
             M, N, K = rnd.choice([1, 1, 2, 4]), rnd.randint(16, 200), rnd.randint(1, 40)
+            if long_k and rnd.random() < 0.5:
+                K = rnd.randint(40, 700)
             if rnd.random() < 0.6:
                 N0 = 16
         elif kind < 0.7:
@@ -131,15 +133,23 @@ def test_mmt4d_random_cases(gpu_lib, oracle_lib):
         os_ = N * M0 * N0 + rnd.choice([0, 0, 4, 16])
         lo, ro, oo = rnd.choice([0, 0, 16, 64]), rnd.choice([0, 0, 32, 128]), rnd.choice([0, 0, 4, 8])
         rng = np.random.default_rng(case)
+        is_f16 = False
         if lb == 8:
             lhs = rng.integers(-128, 128, lo + M * ls, dtype=np.int8)
             rhs = rng.integers(-128, 128, (ro + N * rs) * rb // 8, dtype=np.int8)
             init = rng.integers(-10000, 10000, oo + M * os_, dtype=np.int32)
+        elif lb == 32:
+            lhs = rng.standard_normal(lo + M * ls).astype(np.float32)
+            rhs = (rng.standard_normal(ro + N * rs) / 8).astype(np.float32)
+            init = rng.standard_normal(oo + M * os_).astype(np.float32)
         else:
-            to_bits = synth.f16_bits if typ == abi.MMT4D_TYPE_F16F16F32 else synth.bf16_bits
+            is_f16 = (typ & abi.MMT4D_TYPE_MASK) in (abi.MMT4D_TYPE_F16F16F32, abi.MMT4D_TYPE_F16F16F16)
+            to_bits = synth.f16_bits if is_f16 else synth.bf16_bits
             lhs = to_bits(rng.standard_normal(lo + M * ls).astype(np.float32))
             rhs = to_bits((rng.standard_normal(ro + N * rs) / 8).astype(np.float32))
             init = rng.standard_normal(oo + M * os_).astype(np.float32)
+            if ob == 16:
+                init = to_bits(init)
 
         def params(l, r, o):
             p = abi.Mmt4dParams()
@@ -162,7 +172,31 @@ def test_mmt4d_random_cases(gpu_lib, oracle_lib):
             case, typ, M, N, K, M0, N0, K0, flags, ls, rs, os_, lo, ro, oo, kernel.decode())
         if want.dtype == np.int32:
             assert np.array_equal(got, want), what
-        else:
-            rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
-            assert np.all(np.abs(got - want) <= 1e-3 * np.maximum(np.abs(want), rms)), what
+            continue
+        ulp = 0.0
+        if ob == 16:   # one rounding to the 16-bit output at the end: within one unit in the last place on top
+            got = got.view(np.uint16)
+            if is_f16:
+                got, want, ulp = got.view(np.float16).astype(np.float32), want.view(np.float16).astype(np.float32), 2.0 ** -10
+            else:
+                got, want = (got.astype(np.uint32) << 16).view(np.float32), (want.astype(np.uint32) << 16).view(np.float32)
+                ulp = 2.0 ** -7
+        rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+        assert np.all(np.abs(got - want) <= (1e-3 + ulp) * np.maximum(np.abs(want), rms)), what
+    return kernels
+
+
+def test_mmt4d_random_cases(gpu_lib, oracle_lib):
+    types = [abi.MMT4D_TYPE_S8S8S32, abi.MMT4D_TYPE_S8S4S32, abi.MMT4D_TYPE_F16F16F32, abi.MMT4D_TYPE_BF16BF16F32]
+    kernels = _mmt4d_sweep(gpu_lib, oracle_lib, 1, 300, types, [4, 8, 16, 16], long_k=False)
     assert {b"mmt4d_generic", b"mmt4d_mfma_64x64", b"mmt4d_gemv"} <= kernels
+
+
+def test_mmt4d_random_cases_more_types_and_shapes(gpu_lib, oracle_lib):
+    # f32 and the 16-bit outputs (roundings between k steps skipped) as well, rhs tiles down to 2 rows, and skinny
+    # problems with a K long enough for every wavefront of the narrow-tile kernel to get several rounds.
+    skip = abi.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS
+    types = [abi.MMT4D_TYPE_S8S8S32, abi.MMT4D_TYPE_S8S8S32, abi.MMT4D_TYPE_F16F16F32, abi.MMT4D_TYPE_BF16BF16F32,
+             abi.MMT4D_TYPE_F32F32F32, abi.MMT4D_TYPE_F16F16F16 | skip, abi.MMT4D_TYPE_BF16BF16BF16 | skip]
+    kernels = _mmt4d_sweep(gpu_lib, oracle_lib, 21, 300, types, [2, 4, 8, 16, 16], long_k=True)
+    assert {b"mmt4d_generic", b"mmt4d_mfma_64x64", b"mmt4d_skinny"} <= kernels
