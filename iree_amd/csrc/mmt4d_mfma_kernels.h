@@ -807,7 +807,15 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   const uint8_t* ring_bytes =
       (const uint8_t*)ring + (ROWS16 ? 16 * (64 * ((lane & 31) >> 4) + 16 * (lane >> 5) + (lane & 15))
                                      : (G == 16 ? 16 : G) * lane);
-  const uint32_t pair_a_lane = PAIR_A ? 2 * lane : 0, pair_b_lane = PAIR_B ? 2 * lane : 0;  // dwords, not 16-bit elements
+  // G == 2: lanes address dwords, not 16-bit elements. Paired: dword number
+  // lane; unpaired: the dword that holds the lane's element (two lanes share
+  // it), from which `own_half` then picks the low or the high half. (16-bit
+  // reads that fill the halves of a register one after the other made these
+  // tiles 1.8x slower than the 4-byte ones: the second read of a register has
+  // to wait for the first.)
+  const int32_t pair_a_lane = G != 2 ? 0 : (PAIR_A ? 2 * lane : -2 * (lane & 1));
+  const int32_t pair_b_lane = G != 2 ? 0 : (PAIR_B ? 2 * lane : -2 * (lane & 1));
+  const uint32_t own_half = (lane & 1) ? 0x07060302u : 0x05040100u;
   constexpr int KK16 = ROWS16 ? 32 : 64;
 
   // One pipeline step for the chunk whose fragments are in `cur`:
@@ -844,7 +852,7 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
     // after the read was issued (a wavefront issues in order: splitting right
     // away would stall it, MFMAs included, for the LDS latency of every unit).
     constexpr int SPLIT_DELAY = TAIL_FREE < 3 ? TAIL_FREE : 3;
-    uint2 raw_pair[(PAIR_A || PAIR_B) ? READS : 1];
+    uint2 raw_pair[G == 2 ? READS : 1];
     // Where read unit u of the next step's fragments goes.
     auto unit_of = [&](int u, bool* is_b, bool* paired, int* kk, int* y) {
       *kk = u / (UNITS_A + UNITS_B);
@@ -854,16 +862,19 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
       *y = *is_b ? x : x - UNITS_B;
     };
     auto split_units_of = [&](int read_slot) {
-      if constexpr (PAIR_A || PAIR_B) {
+      if constexpr (G == 2) {
         if (read_slot < 0 || read_slot >= SLOTS) return;
 #pragma unroll
         for (int u = read_slot * READS / SLOTS; u < (read_slot + 1) * READS / SLOTS; ++u) {
           bool is_b, paired;
           int kk, y;
           unit_of(u, &is_b, &paired, &kk, &y);
-          if (!paired) continue;
           uint4(*nxt)[2] = is_b ? nxt_b : nxt_a;
-          split_pair_part(raw_pair[u], y % 4, nxt[2 * (y / 4)][kk], nxt[2 * (y / 4) + 1][kk]);
+          if (paired) {
+            split_pair_part(raw_pair[u], y % 4, nxt[2 * (y / 4)][kk], nxt[2 * (y / 4) + 1][kk]);
+          } else {
+            set_dword(nxt[y / 4][kk], y % 4, __builtin_amdgcn_perm(raw_pair[u].y, raw_pair[u].x, own_half));
+          }
         }
       }
     };
@@ -915,8 +926,9 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
             } else {
               const uint8_t* first = src + 1024 * (2 * frag + kk);
               if constexpr (G == 2) {
-                const uint32_t w = gather_dword(first, part);
-                if (part == 0) dst.x = w; else if (part == 1) dst.y = w; else if (part == 2) dst.z = w; else dst.w = w;
+                // Elements 2*part and 2*part + 1 of the lane's eight, 128 bytes apart, each with its neighbour.
+                raw_pair[u] = make_uint2(*(const uint32_t*)(first + 256 * part), *(const uint32_t*)(first + 256 * part + 128));
+                (void)dst;
               } else if constexpr (G == 8) {
                 // One 64-bit read (two dword reads of adjacent addresses, which
                 // is what the compiler makes of 4-byte aligned accesses, collide
