@@ -626,9 +626,10 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   //     32*h + r of the operand is then row r of fragment f at that k step: the
   //     MFMA operand of lane 32*h + r for K-step kk is elements d = 0 .. 16/G - 1,
   //     each read linear in the lane number (4-byte pieces: two paired dword
-  //     reads; 8-byte: two 64-bit reads; 2-byte: eight 16-bit reads, which
-  //     makes that layout LDS-instruction bound). K is permuted inside a
-  //     chunk, identically for lhs and rhs.
+  //     reads; 8-byte: two 64-bit reads; 2-byte: eight reads of the dword the
+  //     element shares with its neighbour row, and a byte permute that picks
+  //     the lane's half). K is permuted inside a chunk, identically for lhs
+  //     and rhs.
   //   G == 2, fragments in pairs (an even number of them per wavefront): 16-bit
   //     reads deliver half of what the LDS can, so a lane reads dwords, i.e. two
   //     adjacent rows of one k step, and gives the low half to fragment 2p, the
@@ -835,7 +836,7 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
     constexpr int SUB = SubSteps<KIND>::value;
     constexpr int MFMAS = 2 * AM * BN * SUB;
     // Units a fragment's LDS reads are dealt out in: a 128-bit read; two pairs of
-    // dwords; two 64-bit reads; four pairs of 16-bit reads.
+    // dwords; two 64-bit reads; four pairs of dwords holding 16-bit elements.
     constexpr int PARTS = G == 16 ? 1 : (G == 2 ? 4 : 2);
     // Read units, in the order the next step consumes them: per K-step the rhs
     // fragments, then the lhs fragments. An int4 rhs fragment is read once, raw,
