@@ -21,6 +21,13 @@
 // f16f16f16 and bf16bf16bf16 are taken with the flag that skips the roundings
 // between k steps (mmt4d_tile_generic.c:229-286, 319-376): f32 accumulators,
 // one rounding to the 16-bit output at the end.
+//
+// Also here, because nothing else takes them but the generic kernel:
+// s16s16s32 (v_dot2_i32_i16) and s16u4s32, the x86-64 VNNI tile 1x32x8 for
+// 4-bit weights against 16-bit activations (mmt4d_x86_64_tiles.inl; unsigned
+// nibbles, element 2j in the low nibble of byte j, mmt4d_tile_generic.c:108-142):
+// a lane's 16 bytes are 4 rows x 8 nibbles of one k step, each byte is spread
+// to a pair of 16-bit values and multiplied with the matching pair of the lhs.
 #include "uk_device.h"
 #include "uk_internal.h"
 
@@ -29,8 +36,9 @@ namespace {
 
 typedef int v4i32 __attribute__((ext_vector_type(4)));
 typedef _Float16 v2f16 __attribute__((ext_vector_type(2)));
+typedef short v2i16 __attribute__((ext_vector_type(2)));
 
-enum Kind { kI8 = 0, kF16 = 1, kBF16 = 2, kF32 = 3 };
+enum Kind { kI8 = 0, kF16 = 1, kBF16 = 2, kF32 = 3, kI16 = 4, kI16U4 = 5 };
 
 struct SkinnyArgs {
   const uint8_t* lhs;
@@ -47,25 +55,64 @@ struct SkinnyArgs {
 
 template <int KIND> struct Acc { typedef float type; };
 template <> struct Acc<kI8> { typedef int32_t type; };
+template <> struct Acc<kI16> { typedef int32_t type; };
+template <> struct Acc<kI16U4> { typedef int32_t type; };
+// The lhs piece of one k step in registers: G bytes, zero-extended to two
+// dwords; 16 bytes (8 values of 16 bits) against 8 nibbles of the rhs.
+template <int KIND> struct LhsPiece { typedef uint2 type; };
+template <> struct LhsPiece<kI16U4> { typedef uint4 type; };
+
+__device__ __forceinline__ int32_t dot2_i16(uint32_t a, uint32_t b, int32_t c) {
+  return __builtin_amdgcn_sdot2(__builtin_bit_cast(v2i16, a), __builtin_bit_cast(v2i16, b), c, false);
+}
 
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
 __device__ __forceinline__ float f16_lo(uint32_t w) { return (float)__builtin_bit_cast(v2f16, w)[0]; }
 __device__ __forceinline__ float f16_hi(uint32_t w) { return (float)__builtin_bit_cast(v2f16, w)[1]; }
 
-// The lhs piece (G bytes) of one k step, zero-extended into two dwords.
-template <int G>
-__device__ __forceinline__ uint2 load_lhs_piece(const uint8_t* p) {
-  if constexpr (G == 2) return make_uint2(*(const uint16_t*)p, 0);
+template <int KIND, int G>
+__device__ __forceinline__ typename LhsPiece<KIND>::type load_lhs_piece(const uint8_t* p) {
+  if constexpr (KIND == kI16U4) return *(const uint4*)p;
+  else if constexpr (G == 2) return make_uint2(*(const uint16_t*)p, 0);
   else if constexpr (G == 4) return make_uint2(*(const uint32_t*)p, 0);
   else return *(const uint2*)p;
 }
 
 // acc[r] += (row r of the 16 / G rows in `v`) . (lhs piece l), all of one k step.
 template <int KIND, int G>
-__device__ __forceinline__ void multiply_piece(const uint4 v, const uint2 l, typename Acc<KIND>::type* acc) {
+__device__ __forceinline__ void multiply_piece(const uint4 v, const typename LhsPiece<KIND>::type l,
+                                               typename Acc<KIND>::type* acc) {
   const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-  if constexpr (KIND == kI8) {
+  if constexpr (KIND == kI16U4) {
+    static_assert(G == 4, "8 nibbles per row piece");
+    const uint32_t lhs[4] = {l.x, l.y, l.z, l.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        // byte b of the row: its low nibble to bits 0..3, its high nibble to bits 16..19
+        const uint32_t twice = __builtin_amdgcn_perm(0, w[i], 0x0C000C00u + 0x00010001u * b);
+        const uint32_t pair = (twice & 0xFu) | ((twice >> 4) & 0x000F0000u);
+        acc[i] = dot2_i16(pair, lhs[b], acc[i]);
+      }
+    }
+  } else if constexpr (KIND == kI16) {
+    if constexpr (G == 2) {
+      // Two rows per dword: the lhs value in the low resp. high half, zero in the other.
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc[2 * i] = dot2_i16(w[i], l.x, acc[2 * i]);
+        acc[2 * i + 1] = dot2_i16(w[i], l.x << 16, acc[2 * i + 1]);
+      }
+    } else if constexpr (G == 4) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] = dot2_i16(w[i], l.x, acc[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) acc[i] = dot2_i16(w[2 * i + 1], l.y, dot2_i16(w[2 * i], l.x, acc[i]));
+    }
+  } else if constexpr (KIND == kI8) {
     if constexpr (G == 2) {
       // Two rows per dword: the lhs pair in the low resp. high half, zeros in the other.
       const int lo = (int)l.x, hi = (int)(l.x << 16);
@@ -133,7 +180,7 @@ __global__ __launch_bounds__(256) void mmt4d_skinny_kernel(const SkinnyArgs a) {
   static_assert(!NARROW || KIND == kF16 || KIND == kBF16, "16-bit outputs are floats");
   typedef typename Acc<KIND>::type acc_t;
   constexpr int R = 16 / G;  // rhs rows in a lane's 16 bytes
-  __shared__ acc_t partial[4][ROWS][16];
+  __shared__ acc_t partial[4][ROWS][32];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int32_t M0 = 1 << a.log2_M0, N0 = 1 << a.log2_N0;
@@ -142,14 +189,15 @@ __global__ __launch_bounds__(256) void mmt4d_skinny_kernel(const SkinnyArgs a) {
   const int log2_kstep_bytes = a.log2_N0 + (G == 2 ? 1 : (G == 4 ? 2 : 3));
   const int log2_lanes_per_kstep = log2_kstep_bytes - 4;
   const int32_t kstep_in_block = lane >> log2_lanes_per_kstep;
-  const int32_t lhs_kstep_bytes = G << a.log2_M0;
+  constexpr int LHS_G = KIND == kI16U4 ? 16 : G;  // bytes of an lhs row piece
+  const int32_t lhs_kstep_bytes = LHS_G << a.log2_M0;
 
   const uint8_t* rhs_tile = a.rhs + (int64_t)blockIdx.x * a.rhs_stride_bytes;
   const uint8_t* lhs_row[ROWS];
 #pragma unroll
   for (int m = 0; m < ROWS; ++m) {
     const int row = m < a.rows ? m : a.rows - 1;  // clamp: computed, not stored
-    lhs_row[m] = a.lhs + (int64_t)(row >> a.log2_M0) * a.lhs_stride_bytes + (row & (M0 - 1)) * G;
+    lhs_row[m] = a.lhs + (int64_t)(row >> a.log2_M0) * a.lhs_stride_bytes + (row & (M0 - 1)) * LHS_G;
   }
 
   acc_t acc[ROWS][R];
@@ -161,7 +209,7 @@ __global__ __launch_bounds__(256) void mmt4d_skinny_kernel(const SkinnyArgs a) {
   const int64_t blocks = (a.tile_bytes + 1023) >> 10;
   for (int64_t j0 = wave; j0 < blocks; j0 += 4 * UNROLL) {
     uint4 v[UNROLL];
-    uint2 l[UNROLL][ROWS];
+    typename LhsPiece<KIND>::type l[UNROLL][ROWS];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       const int64_t off = ((j0 + 4 * u) << 10) + 16 * lane;
@@ -172,8 +220,8 @@ __global__ __launch_bounds__(256) void mmt4d_skinny_kernel(const SkinnyArgs a) {
       const int64_t kstep = inside ? ((j0 + 4 * u) << (10 - log2_kstep_bytes)) + kstep_in_block : 0;
 #pragma unroll
       for (int m = 0; m < ROWS; ++m) {
-        l[u][m] = load_lhs_piece<G>(lhs_row[m] + kstep * lhs_kstep_bytes);
-        if (!inside) l[u][m] = make_uint2(0, 0);  // 0 * 0, whatever the lhs holds there
+        l[u][m] = load_lhs_piece<KIND, G>(lhs_row[m] + kstep * lhs_kstep_bytes);
+        if (!inside) l[u][m] = typename LhsPiece<KIND>::type{};  // 0 * 0, whatever the lhs holds there
       }
     }
 #pragma unroll
@@ -234,6 +282,8 @@ bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, int* piece_bytes,
     case IREE_UK_FLAG_MMT4D_TYPE_F16F16F32: *kind = kF16; elem_bytes = 2; break;
     case IREE_UK_FLAG_MMT4D_TYPE_BF16BF16F32: *kind = kBF16; elem_bytes = 2; break;
     case IREE_UK_FLAG_MMT4D_TYPE_F32F32F32: *kind = kF32; elem_bytes = 4; break;
+    case IREE_UK_FLAG_MMT4D_TYPE_S16S16S32: *kind = kI16; elem_bytes = 2; break;
+    case IREE_UK_FLAG_MMT4D_TYPE_S16U4S32: *kind = kI16U4; elem_bytes = 2; break;
     case IREE_UK_FLAG_MMT4D_TYPE_F16F16F16:
       if (!skip_roundings) return false;
       *kind = kF16; elem_bytes = 2; *narrow = true;
@@ -244,17 +294,22 @@ bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, int* piece_bytes,
       break;
     default: return false;
   }
-  const int g = a.K0 * elem_bytes;
+  const bool u4 = *kind == kI16U4;
+  if (u4 && a.K0 != 8) return false;
+  const int g = u4 ? 4 : a.K0 * elem_bytes;        // bytes of an rhs row piece
+  const int lhs_g = u4 ? 16 : g;
   if (g != 2 && g != 4 && g != 8) return false;
   const int lm0 = log2_exact(a.M0), ln0 = log2_exact(a.N0);
   // A k step of the rhs must be whole 16-byte vectors.
-  if (lm0 < 0 || ln0 < 0 || a.M0 > 8 || a.N0 > 16 || a.N0 * g < 16) return false;
+  if (lm0 < 0 || ln0 < 0 || a.M0 > 8 || a.N0 > 32 || a.N0 * g < 16) return false;
   *piece_bytes = g;
-  if (probe_only) return a.M0 * g < 16;  // what no matrix kernel takes
+  if (probe_only) return a.M0 * g < 16 || *kind == kI16 || u4;  // what no matrix kernel takes
   if (a.M * a.M0 > 8 || a.M <= 0 || a.K <= 0 || a.N <= 0 || a.N > 0x7FFFFFFF) return false;
-  const int64_t lhs_stride_bytes = a.lhs_stride0 * elem_bytes, rhs_stride_bytes = a.rhs_stride0 * elem_bytes;
+  if (u4 && (a.rhs_stride0 & 1)) return false;
+  const int64_t lhs_stride_bytes = a.lhs_stride0 * elem_bytes;
+  const int64_t rhs_stride_bytes = u4 ? a.rhs_stride0 / 2 : a.rhs_stride0 * elem_bytes;
   if ((uintptr_t)a.rhs % 16 || (a.N > 1 && rhs_stride_bytes % 16)) return false;
-  if ((uintptr_t)a.lhs % g || (a.M > 1 && lhs_stride_bytes % g)) return false;
+  if ((uintptr_t)a.lhs % lhs_g || (a.M > 1 && lhs_stride_bytes % lhs_g)) return false;
   if ((uintptr_t)a.out % (*narrow ? 2 : 4)) return false;
   s->lhs = a.lhs; s->rhs = a.rhs; s->out = a.out;
   s->lhs_stride_bytes = lhs_stride_bytes;
@@ -301,6 +356,8 @@ hipError_t launch_skinny(const Mmt4dArgs& a, hipStream_t stream, const char** na
       return narrow ? launch_kind<kF16, true>(s, piece_bytes, stream) : launch_kind<kF16, false>(s, piece_bytes, stream);
     case kBF16:
       return narrow ? launch_kind<kBF16, true>(s, piece_bytes, stream) : launch_kind<kBF16, false>(s, piece_bytes, stream);
+    case kI16: return launch_kind<kI16, false>(s, piece_bytes, stream);
+    case kI16U4: return launch_piece<kI16U4, 4, false>(s, stream);
     default: return launch_kind<kF32, false>(s, piece_bytes, stream);
   }
 }

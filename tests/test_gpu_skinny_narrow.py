@@ -72,6 +72,46 @@ def test_eight_row_tiles_a_matrix_kernel_can_load_go_there(gpu_lib):
     run_case(gpu_lib, S8, 1, 40, 64, 8, 16, 2, "mmt4d_skinny", offsets=(8, 0, 0))
 
 
+def run_s16_case(gpu_lib, u4, M, N, K, M0, N0, K0, accumulate, expect_kernel, seed=0):
+    """s16s16s32 or s16u4s32 against an exact float64 product (values small enough that no int32 sum wraps)."""
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    lhs = torch.randint(-300, 301, (M * K * M0 * K0,), dtype=torch.int16, device="cuda", generator=g)
+    if u4:
+        packed = torch.randint(0, 256, (N * K * N0 * K0 // 2,), dtype=torch.uint8, device="cuda", generator=g)
+        b = torch.stack([packed & 0xF, packed >> 4], dim=-1).reshape(N, K, N0, K0)  # element 2j in the low nibble of byte j
+        rhs = packed
+    else:
+        rhs = torch.randint(-300, 301, (N * K * N0 * K0,), dtype=torch.int16, device="cuda", generator=g)
+        b = rhs.view(N, K, N0, K0)
+    out = torch.randint(-1000, 1000, (M * N * M0 * N0,), dtype=torch.int32, device="cuda", generator=g)
+    before = out.clone()
+    flags = (abi.MMT4D_TYPE_S16U4S32 if u4 else abi.MMT4D_TYPE_S16S16S32) | (abi.MMT4D_ACCUMULATE if accumulate else 0)
+    p = mm_params(lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), M, N, K, M0, N0, K0, flags)
+    gpu_lib.iree_uk_mmt4d_p(C.byref(p))
+    assert gpu_lib.iree_uk_mi355x_last_kernel() == expect_kernel.encode()
+    a2 = lhs.view(M, K, M0, K0).permute(0, 2, 1, 3).reshape(M * M0, K * K0).double()
+    b2 = b.permute(0, 2, 1, 3).reshape(N * N0, K * K0).double()
+    ref = a2 @ b2.t()
+    if accumulate:
+        ref = ref + before.view(M, N, M0, N0).permute(0, 2, 1, 3).reshape(M * M0, N * N0).double()
+    got = out.view(M, N, M0, N0).permute(0, 2, 1, 3).reshape(M * M0, N * N0)
+    assert torch.equal(got.long(), ref.long())
+
+
+# The x86-64 VNNI tiles for 16-bit activations: s16s16s32 Mx16x2 / Mx8x2 and s16u4s32 1x32x8 (mmt4d_x86_64_tiles.inl).
+@pytest.mark.parametrize("u4,M,M0,N0,K0", [(False, 1, 1, 16, 2), (False, 1, 4, 16, 2), (False, 3, 2, 8, 2), (False, 1, 8, 16, 2),
+                                           (False, 1, 1, 8, 1), (False, 1, 2, 4, 4), (True, 1, 1, 32, 8), (True, 1, 4, 32, 8),
+                                           (True, 5, 1, 16, 8), (True, 1, 2, 4, 8)])
+def test_sixteen_bit_integer_types(gpu_lib, u4, M, M0, N0, K0):
+    for n, K in enumerate((1, 50, 1100)):
+        run_s16_case(gpu_lib, u4, M, 23 + n, K, M0, N0, K0, bool(n & 1), "mmt4d_skinny", seed=K + M0)
+
+
+def test_sixteen_bit_integer_types_with_more_rows_stay_generic(gpu_lib):
+    run_s16_case(gpu_lib, False, 2, 9, 20, 8, 16, 2, True, "mmt4d_generic")
+    run_s16_case(gpu_lib, True, 1, 9, 20, 16, 32, 8, False, "mmt4d_generic")
+
+
 def test_more_rows_than_the_kernel_takes_fall_through(gpu_lib):
     # 9 rows of 1x16x2 int8 tiles: no matrix kernel loads such an lhs either; the generic kernel, still exact.
     run_case(gpu_lib, S8, 9, 20, 40, 1, 16, 2, "mmt4d_generic", accumulate=True)
