@@ -28,6 +28,12 @@
 // nibbles, element 2j in the low nibble of byte j, mmt4d_tile_generic.c:108-142):
 // a lane's 16 bytes are 4 rows x 8 nibbles of one k step, each byte is spread
 // to a pair of 16-bit values and multiplied with the matching pair of the lhs.
+// And s8s4s32 with the Arm tiles Mx8x8 and Mx8x16 (mmt4d_arm_64_tiles.inl;
+// signed nibbles, mmt4d_tile_generic.c:11-51): the even and the odd nibbles of
+// a dword are isolated in the high nibbles of two dwords (int8 values 16 times
+// the weights) and multiplied with the even resp. odd lhs bytes of the k step,
+// which are gathered once per lhs piece; the sums are shifted right by 4 at
+// the end (exact; K * K0 < 131072 keeps 16x the sums inside int32).
 #include "uk_device.h"
 #include "uk_internal.h"
 
@@ -38,7 +44,7 @@ typedef int v4i32 __attribute__((ext_vector_type(4)));
 typedef _Float16 v2f16 __attribute__((ext_vector_type(2)));
 typedef short v2i16 __attribute__((ext_vector_type(2)));
 
-enum Kind { kI8 = 0, kF16 = 1, kBF16 = 2, kF32 = 3, kI16 = 4, kI16U4 = 5 };
+enum Kind { kI8 = 0, kF16 = 1, kBF16 = 2, kF32 = 3, kI16 = 4, kI16U4 = 5, kI8I4 = 6 };
 
 struct SkinnyArgs {
   const uint8_t* lhs;
@@ -57,10 +63,13 @@ template <int KIND> struct Acc { typedef float type; };
 template <> struct Acc<kI8> { typedef int32_t type; };
 template <> struct Acc<kI16> { typedef int32_t type; };
 template <> struct Acc<kI16U4> { typedef int32_t type; };
+template <> struct Acc<kI8I4> { typedef int32_t type; };
 // The lhs piece of one k step in registers: G bytes, zero-extended to two
 // dwords; 16 bytes (8 values of 16 bits) against 8 nibbles of the rhs.
 template <int KIND> struct LhsPiece { typedef uint2 type; };
 template <> struct LhsPiece<kI16U4> { typedef uint4 type; };
+// int4 rhs: per 8 lhs bytes one dword of the even and one of the odd ones.
+template <> struct LhsPiece<kI8I4> { typedef uint4 type; };
 
 __device__ __forceinline__ int32_t dot2_i16(uint32_t a, uint32_t b, int32_t c) {
   return __builtin_amdgcn_sdot2(__builtin_bit_cast(v2i16, a), __builtin_bit_cast(v2i16, b), c, false);
@@ -74,7 +83,17 @@ __device__ __forceinline__ float f16_hi(uint32_t w) { return (float)__builtin_bi
 template <int KIND, int G>
 __device__ __forceinline__ typename LhsPiece<KIND>::type load_lhs_piece(const uint8_t* p) {
   if constexpr (KIND == kI16U4) return *(const uint4*)p;
-  else if constexpr (G == 2) return make_uint2(*(const uint16_t*)p, 0);
+  else if constexpr (KIND == kI8I4) {
+    uint4 raw = make_uint4(0, 0, 0, 0);
+    if constexpr (G == 4) {
+      const uint2 half = *(const uint2*)p;
+      raw.x = half.x; raw.y = half.y;
+    } else {
+      raw = *(const uint4*)p;
+    }
+    return make_uint4(__builtin_amdgcn_perm(raw.y, raw.x, 0x06040200u), __builtin_amdgcn_perm(raw.y, raw.x, 0x07050301u),
+                      __builtin_amdgcn_perm(raw.w, raw.z, 0x06040200u), __builtin_amdgcn_perm(raw.w, raw.z, 0x07050301u));
+  } else if constexpr (G == 2) return make_uint2(*(const uint16_t*)p, 0);
   else if constexpr (G == 4) return make_uint2(*(const uint32_t*)p, 0);
   else return *(const uint2*)p;
 }
@@ -84,7 +103,19 @@ template <int KIND, int G>
 __device__ __forceinline__ void multiply_piece(const uint4 v, const typename LhsPiece<KIND>::type l,
                                                typename Acc<KIND>::type* acc) {
   const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-  if constexpr (KIND == kI16U4) {
+  if constexpr (KIND == kI8I4) {
+    static_assert(G == 4 || G == 8, "8 or 16 nibbles per row piece");
+    const uint32_t lhs[4] = {l.x, l.y, l.z, l.w};
+#pragma unroll
+    for (int i = 0; i < 16 / G; ++i) {
+#pragma unroll
+      for (int d = 0; d < G / 4; ++d) {
+        const uint32_t nibbles = w[i * (G / 4) + d];
+        acc[i] = __builtin_amdgcn_sdot4((int)((nibbles << 4) & 0xF0F0F0F0u), (int)lhs[2 * d], acc[i], false);
+        acc[i] = __builtin_amdgcn_sdot4((int)(nibbles & 0xF0F0F0F0u), (int)lhs[2 * d + 1], acc[i], false);
+      }
+    }
+  } else if constexpr (KIND == kI16U4) {
     static_assert(G == 4, "8 nibbles per row piece");
     const uint32_t lhs[4] = {l.x, l.y, l.z, l.w};
 #pragma unroll
@@ -189,7 +220,7 @@ __global__ __launch_bounds__(256) void mmt4d_skinny_kernel(const SkinnyArgs a) {
   const int log2_kstep_bytes = a.log2_N0 + (G == 2 ? 1 : (G == 4 ? 2 : 3));
   const int log2_lanes_per_kstep = log2_kstep_bytes - 4;
   const int32_t kstep_in_block = lane >> log2_lanes_per_kstep;
-  constexpr int LHS_G = KIND == kI16U4 ? 16 : G;  // bytes of an lhs row piece
+  constexpr int LHS_G = KIND == kI16U4 ? 16 : (KIND == kI8I4 ? 2 * G : G);  // bytes of an lhs row piece
   const int32_t lhs_kstep_bytes = LHS_G << a.log2_M0;
 
   const uint8_t* rhs_tile = a.rhs + (int64_t)blockIdx.x * a.rhs_stride_bytes;
@@ -251,6 +282,7 @@ __global__ __launch_bounds__(256) void mmt4d_skinny_kernel(const SkinnyArgs a) {
     sum += partial[1][m][j0];
     sum += partial[2][m][j0];
     sum += partial[3][m][j0];
+    if constexpr (KIND == kI8I4) sum >>= 4;
     const int64_t index = (int64_t)(m >> a.log2_M0) * a.out_stride0 +
                           ((int64_t)blockIdx.x << (a.log2_M0 + a.log2_N0)) + ((m & (M0 - 1)) << a.log2_N0) + j0;
     if constexpr (NARROW) {
@@ -284,6 +316,7 @@ bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, int* piece_bytes,
     case IREE_UK_FLAG_MMT4D_TYPE_F32F32F32: *kind = kF32; elem_bytes = 4; break;
     case IREE_UK_FLAG_MMT4D_TYPE_S16S16S32: *kind = kI16; elem_bytes = 2; break;
     case IREE_UK_FLAG_MMT4D_TYPE_S16U4S32: *kind = kI16U4; elem_bytes = 2; break;
+    case IREE_UK_FLAG_MMT4D_TYPE_S8S4S32: *kind = kI8I4; elem_bytes = 1; break;
     case IREE_UK_FLAG_MMT4D_TYPE_F16F16F16:
       if (!skip_roundings) return false;
       *kind = kF16; elem_bytes = 2; *narrow = true;
@@ -294,20 +327,23 @@ bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, int* piece_bytes,
       break;
     default: return false;
   }
-  const bool u4 = *kind == kI16U4;
+  const bool u4 = *kind == kI16U4, i4 = *kind == kI8I4;
   if (u4 && a.K0 != 8) return false;
-  const int g = u4 ? 4 : a.K0 * elem_bytes;        // bytes of an rhs row piece
-  const int lhs_g = u4 ? 16 : g;
+  if (i4 && a.K0 != 8 && a.K0 != 16) return false;
+  const int g = u4 ? 4 : (i4 ? a.K0 / 2 : a.K0 * elem_bytes);  // bytes of an rhs row piece
+  const int lhs_g = u4 ? 16 : (i4 ? a.K0 : g);
   if (g != 2 && g != 4 && g != 8) return false;
   const int lm0 = log2_exact(a.M0), ln0 = log2_exact(a.N0);
   // A k step of the rhs must be whole 16-byte vectors.
   if (lm0 < 0 || ln0 < 0 || a.M0 > 8 || a.N0 > 32 || a.N0 * g < 16) return false;
   *piece_bytes = g;
-  if (probe_only) return a.M0 * g < 16 || *kind == kI16 || u4;  // what no matrix kernel takes
+  if (probe_only) return a.M0 * lhs_g < 16 || *kind == kI16 || u4 || (i4 && a.K0 < 16);  // what no matrix kernel takes
+  // 16x-scaled int4 accumulation must not overflow int32.
+  if (i4 && (int64_t)a.K * a.K0 >= 131072) return false;
   if (a.M * a.M0 > 8 || a.M <= 0 || a.K <= 0 || a.N <= 0 || a.N > 0x7FFFFFFF) return false;
-  if (u4 && (a.rhs_stride0 & 1)) return false;
+  if ((u4 || i4) && (a.rhs_stride0 & 1)) return false;
   const int64_t lhs_stride_bytes = a.lhs_stride0 * elem_bytes;
-  const int64_t rhs_stride_bytes = u4 ? a.rhs_stride0 / 2 : a.rhs_stride0 * elem_bytes;
+  const int64_t rhs_stride_bytes = (u4 || i4) ? a.rhs_stride0 / 2 : a.rhs_stride0 * elem_bytes;
   if ((uintptr_t)a.rhs % 16 || (a.N > 1 && rhs_stride_bytes % 16)) return false;
   if ((uintptr_t)a.lhs % lhs_g || (a.M > 1 && lhs_stride_bytes % lhs_g)) return false;
   if ((uintptr_t)a.out % (*narrow ? 2 : 4)) return false;
@@ -358,6 +394,8 @@ hipError_t launch_skinny(const Mmt4dArgs& a, hipStream_t stream, const char** na
       return narrow ? launch_kind<kBF16, true>(s, piece_bytes, stream) : launch_kind<kBF16, false>(s, piece_bytes, stream);
     case kI16: return launch_kind<kI16, false>(s, piece_bytes, stream);
     case kI16U4: return launch_piece<kI16U4, 4, false>(s, stream);
+    case kI8I4:
+      return piece_bytes == 4 ? launch_piece<kI8I4, 4, false>(s, stream) : launch_piece<kI8I4, 8, false>(s, stream);
     default: return launch_kind<kF32, false>(s, piece_bytes, stream);
   }
 }

@@ -107,6 +107,18 @@ def test_sixteen_bit_integer_types(gpu_lib, u4, M, M0, N0, K0):
         run_s16_case(gpu_lib, u4, M, 23 + n, K, M0, N0, K0, bool(n & 1), "mmt4d_skinny", seed=K + M0)
 
 
+# int4 weights in the Arm tiles (s8s4s32 Mx8x8 with dot products, Mx8x16 with i8mm; mmt4d_arm_64_tiles.inl).
+@pytest.mark.parametrize("M,M0,N0,K0", [(1, 1, 8, 8), (1, 2, 8, 8), (1, 4, 8, 8), (1, 8, 8, 8), (1, 1, 8, 16), (1, 4, 8, 16),
+                                        (3, 1, 16, 16), (2, 2, 4, 8)])
+def test_int4_weights_in_narrow_tiles(gpu_lib, M, M0, N0, K0):
+    S8S4 = abi.MMT4D_TYPE_S8S4S32
+    for n, K in enumerate((1, 33, 700)):
+        run_case(gpu_lib, S8S4, M, 29 + n, K, M0, N0, K0, "mmt4d_skinny", accumulate=bool(n & 1), seed=K + K0)
+    # strided with offsets (in 4-bit elements on the rhs side)
+    run_case(gpu_lib, S8S4, M, 21, 40, M0, N0, K0, "mmt4d_skinny", lhs_pad=16, rhs_pad=64, out_pad=4, offsets=(16, 96, 4),
+             accumulate=True, seed=3)
+
+
 def test_sixteen_bit_integer_types_with_more_rows_stay_generic(gpu_lib):
     run_s16_case(gpu_lib, False, 2, 9, 20, 8, 16, 2, True, "mmt4d_generic")
     run_s16_case(gpu_lib, True, 1, 9, 20, 16, 32, 8, False, "mmt4d_generic")
