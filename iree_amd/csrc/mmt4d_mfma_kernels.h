@@ -852,7 +852,8 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
     // Paired fragments: the dwords of a read unit are split this many MFMAs
     // after the read was issued (a wavefront issues in order: splitting right
     // away would stall it, MFMAs included, for the LDS latency of every unit).
-    constexpr int SPLIT_DELAY = TAIL_FREE < 3 ? TAIL_FREE : 3;
+    // (3 MFMAs: int8 16x16x2 at 4096^3 86 us; 5: 81 us; 8, all there are on the 256x256 tile: 79 us.)
+    constexpr int SPLIT_DELAY = TAIL_FREE;
     uint2 raw_pair[G == 2 ? READS : 1];
     // Where read unit u of the next step's fragments goes.
     auto unit_of = [&](int u, bool* is_b, bool* paired, int* kk, int* y) {
