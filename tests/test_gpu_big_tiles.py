@@ -217,6 +217,31 @@ def test_direct_kernel_with_K_ending_inside_a_chunk(gpu_lib, flags, M0, N0, K0, 
         run_case(gpu_lib, flags, 72 // M0, 88 // N0, K, M0, N0, K0, "mmt4d_mfma_64x64", accumulate=True, seed=K + 100)
 
 
+def test_K_tail_overlap_is_zeroed_in_both_operands(gpu_lib):
+    # The chunk that K ends in is loaded overlapping the one before it. An infinity inside the overlap must count
+    # once: were only one operand zeroed there, inf * 0 would turn the outputs into NaN.
+    M, N, K, M0, N0, K0 = 5, 6, 5, 16, 16, 16      # 32-byte row pieces: chunks [k0,k1], [k2,k3], tail k4 -> the last chunk is [k3,k4]
+    g = torch.Generator(device="cuda").manual_seed(1)
+    lhs = (torch.rand(M * K * M0 * K0, device="cuda", generator=g) + 0.5).to(torch.float16)
+    rhs = (torch.rand(N * K * N0 * K0, device="cuda", generator=g) + 0.5).to(torch.float16)
+    lhs.view(M, K, M0, K0)[0, 3, 0, 7] = float("inf")      # logical row 0, k step 3
+    rhs.view(N, K, N0, K0)[1, 3, 5, 2] = float("inf")      # logical column 21, k step 3
+    out = torch.zeros(M * N * M0 * N0, device="cuda")
+    p = mm_params(lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), M, N, K, M0, N0, K0, abi.MMT4D_TYPE_F16F16F32)
+    gpu_lib.iree_uk_mmt4d_p(C.byref(p))
+    assert gpu_lib.iree_uk_mi355x_last_kernel() == b"mmt4d_mfma_64x64"
+    got = out.view(M, N, M0, N0).permute(0, 2, 1, 3).reshape(M * M0, N * N0)
+    assert not bool(torch.isnan(got).any())
+    inf = torch.isinf(got)
+    want = torch.zeros_like(inf)
+    want[0, :] = True
+    want[:, 21] = True
+    assert torch.equal(inf, want)
+    finite = got[1:, :21]
+    ref = logical(lhs, M, K, M0, K0)[1:] @ logical(rhs, N, K, N0, K0)[:21].t()
+    assert bool(((finite.double() - ref).abs() <= REL_TOL * ref.abs()).all())
+
+
 def test_ragged_K_on_the_register_staged_kernel(gpu_lib):
     # 4-byte aligned rows (not 16): the register-staged kernel with its zero-filling tail step.
     run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, 451, 463, 37, 8, 8, 4, "mmt4d_mfma_256x256", lhs_pad=4, rhs_pad=12,
