@@ -1041,6 +1041,209 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
                                                             first_col + wave_n * (32 * BN), lane);
 }
 
+// (Overloads on scalars rather than a bit cast of a vector element.)
+__device__ __forceinline__ uint32_t value_bits(int32_t v) { return (uint32_t)v; }
+__device__ __forceinline__ uint32_t value_bits(float v) { return __float_as_uint(v); }
+__device__ __forceinline__ void set_from_bits(int32_t& v, uint32_t bits) { v = (int32_t)bits; }
+__device__ __forceinline__ void set_from_bits(float& v, uint32_t bits) { v = __uint_as_float(bits); }
+
+// ---------------------------------------------------------------------------
+// A 64x64 block tile whose four wavefronts split K instead of the tile, for
+// problems with few block tiles and a long K (say 128 x 4096 x 14336: 128
+// tiles). There the kernel above is bound by the latency of one pipeline step
+// (counter wait, barrier, LDS reads; about 140 ns) per 64 bytes of K per
+// workgroup, and half the compute units have no workgroup at all. Here a step
+// covers 256 bytes of K per row: wavefront w multiplies bytes 64*w .. 64*w + 63
+// of every row for the whole tile (2 x 2 fragments), so a workgroup streams
+// four times as much per step, and the four partial tiles are summed through
+// LDS at the end, in wavefront order (deterministic). Row pieces of 16 bytes or
+// more, K a multiple of 256 bytes per row, int8 / f16 / bf16. Measured:
+// 128 x 4096 x 14336 bf16 62 -> 41 us, int8 30 us. What bounds it now is what a
+// compute unit's load path moves (32 KiB per step in about 500 cycles, of a
+// peak of 64 bytes per cycle) on the 64 or 128 compute units that have a tile.
+//
+// LDS stage: per operand four slices (one per wavefront's share of K) of 256
+// 16-byte slots in the layout of the kernel above (G == 16): slot p of a slice
+// holds fragment p >> 7, rows 16*((p >> 6) & 1) + (p & 15), 16-byte column
+// (p >> 4) & 3. Load t of wavefront w fills slots 64*w .. 64*w + 63 of slice t:
+// rows 16*w .. 16*w + 15 of the tile, bytes 64*t .. 64*t + 63 of the chunk.
+template <int KIND, bool NARROW>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2)))
+void mmt4d_mfma_split_k_kernel(const MfmaArgs a) {
+  typedef typename AccType<KIND>::type acc_t;
+  static_assert(KIND != kF32, "one MFMA per fragment pair");
+  constexpr int STAGES = 4, AHEAD = STAGES - 1;  // (a fifth stage, all the LDS there is, changed nothing)
+  constexpr int OPERAND_PIECES = 64 * 16;  // 64 rows x 256 bytes
+  constexpr uint32_t STAGE_BYTES = 2 * OPERAND_PIECES * 16, RING_BYTES = STAGES * STAGE_BYTES;
+  constexpr int LOADS = 8;  // per wavefront and chunk, four of each operand
+
+  int tile_row, tile_col;
+  if (!locate_block(a, &tile_row, &tile_col)) return;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  const int64_t total_rows = (int64_t)a.M << a.log2_M0;
+  const int64_t total_cols = (int64_t)a.N << a.log2_N0;
+  const int64_t lhs_kstep = (int64_t)a.lhs_rb << a.log2_M0;
+  const int64_t rhs_kstep = (int64_t)a.rhs_rb << a.log2_N0;
+  const int64_t lhs_chunk_bytes = (256 >> a.log2_lhs_rb) * lhs_kstep;
+  const int64_t rhs_chunk_bytes = (256 >> a.log2_rhs_rb) * rhs_kstep;
+  const int64_t first_row = (int64_t)tile_row * 64, first_col = (int64_t)tile_col * 64;
+  const uint8_t* lhs_base = a.lhs + (first_row >> a.log2_M0) * a.lhs_stride_bytes;
+  const uint8_t* rhs_base = a.rhs + (first_col >> a.log2_N0) * a.rhs_stride_bytes;
+
+  // Rows past the end of the matrix are redirected to its last row: computed, never stored.
+  auto piece_offset = [&](int64_t row, int64_t last, int64_t first, int log2_t0, int64_t stride_bytes, int32_t rb,
+                          int log2_rb, int64_t kstep, int byte_in_chunk) -> uint32_t {
+    row = min(row, last);
+    const int64_t tile = (row >> log2_t0) - (first >> log2_t0);
+    return (uint32_t)(tile * stride_bytes + (row & ((1 << log2_t0) - 1)) * rb + (byte_in_chunk >> log2_rb) * kstep +
+                      (byte_in_chunk & (rb - 1)));
+  };
+  uint32_t a_off[4], b_off[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int row = 16 * wave + (lane & 15), byte_in_chunk = 64 * t + 16 * (lane >> 4);
+    a_off[t] = piece_offset(first_row + row, total_rows - 1, first_row, a.log2_M0, a.lhs_stride_bytes, a.lhs_rb,
+                            a.log2_lhs_rb, lhs_kstep, byte_in_chunk);
+    b_off[t] = piece_offset(first_col + row, total_cols - 1, first_col, a.log2_N0, a.rhs_stride_bytes, a.rhs_rb,
+                            a.log2_rhs_rb, rhs_kstep, byte_in_chunk);
+  }
+
+  acc_t acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+
+  const int chunks = (int)((((int64_t)a.K << a.log2_lhs_rb)) >> 8);  // whole chunks of 256 bytes per row
+  const int last_chunk = chunks - 1;
+
+  auto issue_load = [&](int n, uint32_t stage_off, const uint8_t* la, const uint8_t* lb) {
+    const bool is_a = n < 4;
+    const int t = n & 3;
+    load_to_lds(stage_off + (is_a ? 0 : OPERAND_PIECES * 16) + (256 * t + 64 * wave) * 16, is_a ? a_off[t] : b_off[t],
+                is_a ? la : lb);
+  };
+  // This wavefront's operand registers for one chunk: fragment f, K-step kk.
+  uint4 pa[2][2], pb[2][2], qa[2][2], qb[2][2];
+  const uint8_t* lane_bytes = (const uint8_t*)ring + 16 * (256 * wave + 64 * ((lane & 31) >> 4) + 16 * (lane >> 5) + (lane & 15));
+
+  const uint8_t* load_a = lhs_base + min(AHEAD, last_chunk) * lhs_chunk_bytes;
+  const uint8_t* load_b = rhs_base + min(AHEAD, last_chunk) * rhs_chunk_bytes;
+  int load_chunk = AHEAD;
+  uint32_t load_stage_off = AHEAD * STAGE_BYTES % RING_BYTES;
+  uint32_t read_stage_off = STAGE_BYTES;
+
+  // One step, as in the kernel above: two MFMAs ahead of the wait and the barrier, then the loads of the chunk
+  // three ahead and the LDS reads of the next chunk dealt out over four MFMAs, two MFMAs without memory work.
+  auto step = [&](const uint4 (*cur_a)[2], const uint4 (*cur_b)[2], uint4 (*nxt_a)[2], uint4 (*nxt_b)[2]) {
+    auto multiply = [&](int m) {
+      const int kk = m >> 2, i = (m >> 1) & 1, j = m & 1;
+      acc[i][j] = mfma<KIND>(cur_b[j][kk], cur_a[i][kk], acc[i][j]);
+    };
+    multiply(0);
+    multiply(1);
+    __builtin_amdgcn_sched_barrier(0);
+    wait_loads_but<LOADS*(AHEAD - 2)>();
+    __builtin_amdgcn_s_barrier();
+    const uint8_t* read_a = lane_bytes + read_stage_off;
+    const uint8_t* read_b = read_a + OPERAND_PIECES * 16;
+#pragma unroll
+    for (int m = 2; m < 8; ++m) {
+      const int slot = m - 2;
+      if (slot < 4) {
+        issue_load(2 * slot, load_stage_off, load_a, load_b);
+        issue_load(2 * slot + 1, load_stage_off, load_a, load_b);
+        __builtin_amdgcn_sched_barrier(0);
+        // Read order: K-step 0 (rhs, lhs), then K-step 1: what the next step consumes first comes first.
+        const int kk = slot >> 1;
+        if ((slot & 1) == 0) {
+          nxt_b[0][kk] = *(const uint4*)(read_b + (32 * kk) * 16);
+          nxt_b[1][kk] = *(const uint4*)(read_b + (128 + 32 * kk) * 16);
+        } else {
+          nxt_a[0][kk] = *(const uint4*)(read_a + (32 * kk) * 16);
+          nxt_a[1][kk] = *(const uint4*)(read_a + (128 + 32 * kk) * 16);
+        }
+      }
+      multiply(m);
+      if (m == 7) {
+        const bool more = load_chunk < last_chunk;
+        load_a += more ? lhs_chunk_bytes : 0;
+        load_b += more ? rhs_chunk_bytes : 0;
+        ++load_chunk;
+        load_stage_off = load_stage_off + STAGE_BYTES == RING_BYTES ? 0 : load_stage_off + STAGE_BYTES;
+        read_stage_off = read_stage_off + STAGE_BYTES == RING_BYTES ? 0 : read_stage_off + STAGE_BYTES;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+#pragma unroll
+  for (int c = 0; c < AHEAD; ++c) {
+    const int idx = min(c, last_chunk);
+#pragma unroll
+    for (int n = 0; n < LOADS; ++n)
+      issue_load(n, (uint32_t)c * STAGE_BYTES, lhs_base + idx * lhs_chunk_bytes, rhs_base + idx * rhs_chunk_bytes);
+  }
+  wait_loads_but<(AHEAD - 1) * LOADS>();
+  __syncthreads();
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+    for (int f = 0; f < 2; ++f) {
+      pb[f][kk] = *(const uint4*)(lane_bytes + (OPERAND_PIECES + 128 * f + 32 * kk) * 16);
+      pa[f][kk] = *(const uint4*)(lane_bytes + (128 * f + 32 * kk) * 16);
+    }
+  int kc = 0;
+  for (; kc + 1 < chunks; kc += 2) {
+    step(pa, pb, qa, qb);
+    step(qa, qb, pa, pb);
+  }
+  if (kc < chunks) step(pa, pb, qa, qb);
+  wait_loads_but<0>();
+  __syncthreads();  // nobody reads operands from the ring any more
+
+  // The four partial tiles, summed in wavefront order. Quadrant q = 2*i + j of the tile ends up with wavefront q;
+  // partial[(q*4 + w)*16 + v][lane] is accumulator register v of wavefront w's fragment (i, j).
+  uint32_t* partial = (uint32_t*)ring;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    if (q != wave) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const typename AccType<KIND>::scalar value = acc[q >> 1][q & 1][v];
+        partial[((q * 4 + wave) * 16 + v) * 64 + lane] = value_bits(value);
+      }
+    }
+  }
+  __syncthreads();
+  acc_t total[1][1];
+  {
+    // (selected without indexing the accumulator array by a run-time value)
+    const acc_t own = wave == 0 ? acc[0][0] : (wave == 1 ? acc[0][1] : (wave == 2 ? acc[1][0] : acc[1][1]));
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      acc_t part;
+      if (w == wave) {
+        part = own;
+      } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          typename AccType<KIND>::scalar value;
+          set_from_bits(value, partial[((wave * 4 + w) * 16 + v) * 64 + lane]);
+          part[v] = value;
+        }
+      }
+      if (w == 0) total[0][0] = part; else total[0][0] += part;
+    }
+  }
+  store_block<KIND, false, NARROW, 1, 1>(a, total, first_row + 32 * (wave >> 1), first_col + 32 * (wave & 1), lane);
+}
+
 // Whether the direct-to-LDS kernel covers the problem: every lane can load 16
 // contiguous bytes (4-byte row pieces 4 rows at a time, an int4 rhs in pieces
 // of 32 nibbles), and K is long enough.
@@ -1080,6 +1283,25 @@ hipError_t launch_direct(MfmaArgs m, hipStream_t stream) {
         hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (attr != hipSuccess) return attr;
   }
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds_bytes, stream, m);
+  return hipGetLastError();
+}
+
+// The 64x64 tile with K split over the wavefronts: few block tiles, a long K that is whole steps of 256 bytes.
+inline bool split_k_pays(const MfmaArgs& m) {
+  const int64_t rows = (int64_t)m.M << m.log2_M0, cols = (int64_t)m.N << m.log2_N0;
+  const int64_t row_bytes = (int64_t)m.K * m.lhs_rb;
+  return ((rows + 63) / 64) * ((cols + 63) / 64) <= 128 && row_bytes % 256 == 0 && row_bytes >= 4096;
+}
+
+template <int KIND, bool NARROW>
+hipError_t launch_split_k(MfmaArgs m, hipStream_t stream) {
+  unsigned grid;
+  set_tile_grid(&m, 64, 64, &grid);
+  constexpr int lds_bytes = 4 * 2 * 64 * 256;
+  auto kernel = mmt4d_mfma_split_k_kernel<KIND, NARROW>;
+  const hipError_t attr = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+  if (attr != hipSuccess) return attr;
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds_bytes, stream, m);
   return hipGetLastError();
 }
@@ -1151,6 +1373,12 @@ int choose_tile(const MfmaArgs& m, bool direct, const TileChoice** chosen) {
 template <int KIND, bool RHS_I4, int G, bool NARROW>
 hipError_t launch_variant(const MfmaArgs& m, hipStream_t stream, const char** name) {
   const bool direct = direct_covers<RHS_I4, G>(m);
+  if constexpr (G == 16 && !RHS_I4 && KIND != kF32) {
+    if (direct && split_k_pays(m)) {
+      *name = "mmt4d_mfma_64x64_split_k";
+      return launch_split_k<KIND, NARROW>(m, stream);
+    }
+  }
   const TileChoice* tile;
   switch (choose_tile<RHS_I4>(m, direct, &tile)) {
     case 0:

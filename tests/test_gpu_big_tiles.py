@@ -242,6 +242,25 @@ def test_K_tail_overlap_is_zeroed_in_both_operands(gpu_lib):
     assert bool(((finite.double() - ref).abs() <= REL_TOL * ref.abs()).all())
 
 
+# Few block tiles against a long K: the 64x64 tile whose wavefronts split K (256 bytes of K per row and step) and sum
+# their partial tiles at the end. Even and odd numbers of steps, ragged tiles, one tile only, accumulation, strides.
+@pytest.mark.parametrize("flags,M0,N0,K0", [(abi.MMT4D_TYPE_S8S8S32, 16, 16, 64), (abi.MMT4D_TYPE_S8S8S32, 8, 8, 16),
+                                            (abi.MMT4D_TYPE_S8S8S32, 4, 16, 32), (abi.MMT4D_TYPE_F16F16F32, 16, 16, 16),
+                                            (abi.MMT4D_TYPE_BF16BF16F32, 16, 16, 8), (abi.MMT4D_TYPE_BF16BF16F32, 1, 16, 8),
+                                            (abi.MMT4D_TYPE_F16F16F16, 16, 16, 8), (abi.MMT4D_TYPE_BF16BF16BF16, 8, 16, 16)])
+def test_split_k_tile(gpu_lib, flags, M0, N0, K0):
+    e = 1 if flags == abi.MMT4D_TYPE_S8S8S32 else 2
+    per_step = 256 // (K0 * e)                      # k steps per 256 bytes of a row
+    name = "mmt4d_mfma_64x64_split_k"
+    run_case(gpu_lib, flags, 72 // M0 + 1, 88 // N0, 16 * per_step, M0, N0, K0, name, accumulate=True, out_pad=8, seed=1)
+    run_case(gpu_lib, flags, 200 // M0, 300 // N0, 17 * per_step, M0, N0, K0, name, lhs_pad=64 // e, rhs_pad=32 // e,
+             offsets=(16 // e, 48 // e, 4), seed=2)
+    run_case(gpu_lib, flags, max(1, 16 // M0), 48 // N0, 41 * per_step, M0, N0, K0, name, accumulate=True, seed=3)
+    # K not whole steps of 256 bytes, or too short to matter: the ordinary 64x64 tile
+    run_case(gpu_lib, flags, 72 // M0 + 1, 88 // N0, 16 * per_step + 64 // (K0 * e), M0, N0, K0, "mmt4d_mfma_64x64", seed=4)
+    run_case(gpu_lib, flags, 72 // M0 + 1, 88 // N0, 8 * per_step, M0, N0, K0, "mmt4d_mfma_64x64", seed=5)
+
+
 def test_ragged_K_on_the_register_staged_kernel(gpu_lib):
     # 4-byte aligned rows (not 16): the register-staged kernel with its zero-filling tail step.
     run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, 451, 463, 37, 8, 8, 4, "mmt4d_mfma_256x256", lhs_pad=4, rhs_pad=12,
