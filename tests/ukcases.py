@@ -159,7 +159,7 @@ MMT4D_TILES_X86 = (
     + _tiles(abi.MMT4D_TYPE_S8S8S32, 16, 16, 2) + _tiles(abi.MMT4D_TYPE_S16S16S32, 16, 16, 2)
     + _tiles(abi.MMT4D_TYPE_BF16BF16F32, 16, 16, 2) + _tiles(abi.MMT4D_TYPE_BF16BF16BF16 | SKIP, 16, 16, 2)
     + _tiles(abi.MMT4D_TYPE_S16U4S32, 1, 32, 8))
-# Tile shapes of this library's specialised GPU kernels (the BASELINE configs).
+# Tile shapes of this library's specialised GPU kernels (the benchmark configurations).
 MMT4D_TILES_GPU = (
     _tiles(abi.MMT4D_TYPE_S8S8S32, 8, 8, 4) + _tiles(abi.MMT4D_TYPE_F16F16F32, 16, 16, 16)
     + _tiles(abi.MMT4D_TYPE_BF16BF16F32, 16, 16, 8) + _tiles(abi.MMT4D_TYPE_S8S4S32, 16, 16, 32)
@@ -248,7 +248,7 @@ PACK_TILES_X86 = [(abi.PACK_TYPE_F32F32, 8, 1), (abi.PACK_TYPE_I8I8, 8, 2),
                   (abi.PACK_TYPE_F32F32, 16, 1), (abi.PACK_TYPE_BF16BF16, 16, 2),
                   (abi.PACK_TYPE_I8I8, 16, 2), (abi.PACK_TYPE_F32F32, 16, 16),
                   (abi.PACK_TYPE_I32I32, 16, 16)]
-# Operand layouts of the BASELINE mmt4d configs.
+# Operand layouts of the benchmark's mmt4d configurations.
 PACK_TILES_GPU = [(abi.PACK_TYPE_I8I8, 8, 4), (abi.PACK_TYPE_F16F16, 16, 16),
                   (abi.PACK_TYPE_BF16BF16, 16, 8), (abi.PACK_TYPE_I8I8, 16, 32),
                   (abi.PACK_TYPE_BF16BF16, 1, 8), (abi.PACK_TYPE_I32I32, 8, 8)]
