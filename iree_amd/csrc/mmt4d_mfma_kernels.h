@@ -1048,34 +1048,46 @@ __device__ __forceinline__ void set_from_bits(int32_t& v, uint32_t bits) { v = (
 __device__ __forceinline__ void set_from_bits(float& v, uint32_t bits) { v = __uint_as_float(bits); }
 
 // ---------------------------------------------------------------------------
-// A 64x64 block tile whose four wavefronts split K instead of the tile, for
-// problems with few block tiles and a long K (say 128 x 4096 x 14336: 128
-// tiles). There the kernel above is bound by the latency of one pipeline step
-// (counter wait, barrier, LDS reads; about 140 ns) per 64 bytes of K per
-// workgroup, and half the compute units have no workgroup at all. Here a step
-// covers 256 bytes of K per row: wavefront w multiplies bytes 64*w .. 64*w + 63
-// of every row for the whole tile (2 x 2 fragments), so a workgroup streams
-// four times as much per step, and the four partial tiles are summed through
-// LDS at the end, in wavefront order (deterministic). Row pieces of 16 bytes or
-// more, K a multiple of 256 bytes per row, int8 / f16 / bf16. Measured:
-// 128 x 4096 x 14336 bf16 62 -> 41 us, int8 30 us. What bounds it now is what a
-// compute unit's load path moves (32 KiB per step in about 500 cycles, of a
-// peak of 64 bytes per cycle) on the 64 or 128 compute units that have a tile.
+// Block tiles whose four wavefronts split K instead of the tile, for problems
+// with few block tiles: few rhs rows against a long K (say 128 x 4096 x 14336,
+// 128 tiles of 64x64), or at most 128 lhs rows (one tile row of 128x64). There
+// the kernel above is bound by the latency of one pipeline step (counter wait,
+// barrier, LDS reads; about 140 ns) per 64 bytes of K per workgroup, and with
+// few tiles half the compute units have no workgroup at all. Here every
+// wavefront multiplies the whole tile ((32*AMF) x 64, AMF x 2 fragments) over
+// its quarter of the step's K bytes, so a workgroup streams more per step, and
+// the four partial tiles are summed through LDS at the end, in wavefront order
+// (deterministic). Row pieces of 16 bytes or more, int8 / f16 / bf16.
+//   AMF == 2: 64x64 tile, 256 bytes of K per row and step (two MFMA K-steps per
+//     wavefront), ring of 4 stages of 32 KiB. 128 x 4096 x 14336 bf16 62 -> 41 us.
+//   AMF == 4: 128x64 tile, 128 bytes of K per row and step (one K-step per
+//     wavefront), ring of 6 stages of 24 KiB.
+// What bounds them is what a compute unit's load path moves (64 bytes per
+// cycle at best; a stage takes about 500 resp. 400 cycles).
 //
-// LDS stage: per operand four slices (one per wavefront's share of K) of 256
-// 16-byte slots in the layout of the kernel above (G == 16): slot p of a slice
-// holds fragment p >> 7, rows 16*((p >> 6) & 1) + (p & 15), 16-byte column
-// (p >> 4) & 3. Load t of wavefront w fills slots 64*w .. 64*w + 63 of slice t:
-// rows 16*w .. 16*w + 15 of the tile, bytes 64*t .. 64*t + 63 of the chunk.
-template <int KIND, bool NARROW>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2)))
+// LDS stage: per operand four slices (one per wavefront's share of K, 16*COLS
+// bytes per row, COLS = 2 * K-steps per wavefront) of fragments in the layout
+// of the kernel above (G == 16) with COLS 16-byte columns: slot p of a
+// fragment holds rows 16*(p / (16*COLS)) + (p & 15), column (p >> 4) & (COLS-1).
+// A load fills 64 consecutive slots of one slice.
+template <int KIND, bool NARROW, int AMF>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, AMF == 2 ? 2 : 1)))
 void mmt4d_mfma_split_k_kernel(const MfmaArgs a) {
   typedef typename AccType<KIND>::type acc_t;
   static_assert(KIND != kF32, "one MFMA per fragment pair");
-  constexpr int STAGES = 4, AHEAD = STAGES - 1;  // (a fifth stage, all the LDS there is, changed nothing)
-  constexpr int OPERAND_PIECES = 64 * 16;  // 64 rows x 256 bytes
-  constexpr uint32_t STAGE_BYTES = 2 * OPERAND_PIECES * 16, RING_BYTES = STAGES * STAGE_BYTES;
-  constexpr int LOADS = 8;  // per wavefront and chunk, four of each operand
+  static_assert(AMF == 2 || AMF == 4, "64 or 128 lhs rows");
+  constexpr int KKW = AMF == 2 ? 2 : 1;       // MFMA K-steps per wavefront and step
+  constexpr int COLS = 2 * KKW;               // 16-byte columns of a slice
+  constexpr int CHUNK_BYTES = 4 * 16 * COLS;  // of K per row and step
+  constexpr int STAGES = AMF == 2 ? 4 : 6, AHEAD = STAGES - 1;  // (a fifth stage of the 64x64 tile changed nothing)
+  constexpr int FRAG_SLOTS = 32 * COLS;
+  constexpr int A_SLICE = AMF * FRAG_SLOTS, B_SLICE = 2 * FRAG_SLOTS;  // slots per slice
+  constexpr int A_PIECES = 4 * A_SLICE, B_PIECES = 4 * B_SLICE;
+  constexpr uint32_t STAGE_BYTES = (A_PIECES + B_PIECES) * 16, RING_BYTES = STAGES * STAGE_BYTES;
+  constexpr int A_LOADS = A_PIECES / 256, B_LOADS = B_PIECES / 256, LOADS = A_LOADS + B_LOADS;  // per wavefront
+  constexpr int READS = KKW * (AMF + 2);      // 128-bit LDS reads per wavefront and step
+  constexpr int MFMAS = KKW * AMF * 2;
+  static_assert(MFMAS == 8 && LOADS <= 8 && READS <= 8, "the step below deals memory work over four of eight MFMAs");
 
   int tile_row, tile_col;
   if (!locate_block(a, &tile_row, &tile_col)) return;
@@ -1087,9 +1099,9 @@ void mmt4d_mfma_split_k_kernel(const MfmaArgs a) {
   const int64_t total_cols = (int64_t)a.N << a.log2_N0;
   const int64_t lhs_kstep = (int64_t)a.lhs_rb << a.log2_M0;
   const int64_t rhs_kstep = (int64_t)a.rhs_rb << a.log2_N0;
-  const int64_t lhs_chunk_bytes = (256 >> a.log2_lhs_rb) * lhs_kstep;
-  const int64_t rhs_chunk_bytes = (256 >> a.log2_rhs_rb) * rhs_kstep;
-  const int64_t first_row = (int64_t)tile_row * 64, first_col = (int64_t)tile_col * 64;
+  const int64_t lhs_chunk_bytes = (CHUNK_BYTES >> a.log2_lhs_rb) * lhs_kstep;
+  const int64_t rhs_chunk_bytes = (CHUNK_BYTES >> a.log2_rhs_rb) * rhs_kstep;
+  const int64_t first_row = (int64_t)tile_row * (32 * AMF), first_col = (int64_t)tile_col * 64;
   const uint8_t* lhs_base = a.lhs + (first_row >> a.log2_M0) * a.lhs_stride_bytes;
   const uint8_t* rhs_base = a.rhs + (first_col >> a.log2_N0) * a.rhs_stride_bytes;
 
@@ -1101,36 +1113,59 @@ void mmt4d_mfma_split_k_kernel(const MfmaArgs a) {
     return (uint32_t)(tile * stride_bytes + (row & ((1 << log2_t0) - 1)) * rb + (byte_in_chunk >> log2_rb) * kstep +
                       (byte_in_chunk & (rb - 1)));
   };
-  uint32_t a_off[4], b_off[4];
+  // Load t of wavefront w is group 4*t + w of its operand's groups of 64 slots, slice by slice.
+  auto group_of = [&](int t, int slice_slots, int* slice, int* row, int* byte_in_chunk) {
+    const int group = 4 * t + wave, per_slice = slice_slots / 64;
+    *slice = group / per_slice;
+    const int p = 64 * (group % per_slice) + lane;  // slot within the slice
+    *row = 32 * (p / FRAG_SLOTS) + 16 * ((p / (16 * COLS)) & 1) + (p & 15);
+    *byte_in_chunk = 16 * COLS * *slice + 16 * ((p >> 4) & (COLS - 1));
+  };
+  uint32_t a_off[A_LOADS], b_off[B_LOADS], a_lds[A_LOADS], b_lds[B_LOADS];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    const int row = 16 * wave + (lane & 15), byte_in_chunk = 64 * t + 16 * (lane >> 4);
+  for (int t = 0; t < A_LOADS; ++t) {
+    int slice, row, byte_in_chunk;
+    group_of(t, A_SLICE, &slice, &row, &byte_in_chunk);
     a_off[t] = piece_offset(first_row + row, total_rows - 1, first_row, a.log2_M0, a.lhs_stride_bytes, a.lhs_rb,
                             a.log2_lhs_rb, lhs_kstep, byte_in_chunk);
+    a_lds[t] = (uint32_t)(64 * (4 * t + wave)) * 16;
+  }
+#pragma unroll
+  for (int t = 0; t < B_LOADS; ++t) {
+    int slice, row, byte_in_chunk;
+    group_of(t, B_SLICE, &slice, &row, &byte_in_chunk);
     b_off[t] = piece_offset(first_col + row, total_cols - 1, first_col, a.log2_N0, a.rhs_stride_bytes, a.rhs_rb,
                             a.log2_rhs_rb, rhs_kstep, byte_in_chunk);
+    b_lds[t] = (uint32_t)(A_PIECES + 64 * (4 * t + wave)) * 16;
   }
 
-  acc_t acc[2][2];
+  acc_t acc[AMF][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < AMF; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
 
-  const int chunks = (int)((((int64_t)a.K << a.log2_lhs_rb)) >> 8);  // whole chunks of 256 bytes per row
+  const int chunks = (int)(((int64_t)a.K << a.log2_lhs_rb) / CHUNK_BYTES);  // K is whole steps
   const int last_chunk = chunks - 1;
 
   auto issue_load = [&](int n, uint32_t stage_off, const uint8_t* la, const uint8_t* lb) {
-    const bool is_a = n < 4;
-    const int t = n & 3;
-    load_to_lds(stage_off + (is_a ? 0 : OPERAND_PIECES * 16) + (256 * t + 64 * wave) * 16, is_a ? a_off[t] : b_off[t],
-                is_a ? la : lb);
+    if (n < A_LOADS) load_to_lds(stage_off + a_lds[n], a_off[n], la);
+    else load_to_lds(stage_off + b_lds[n - A_LOADS], b_off[n - A_LOADS], lb);
   };
   // This wavefront's operand registers for one chunk: fragment f, K-step kk.
-  uint4 pa[2][2], pb[2][2], qa[2][2], qb[2][2];
-  const uint8_t* lane_bytes = (const uint8_t*)ring + 16 * (256 * wave + 64 * ((lane & 31) >> 4) + 16 * (lane >> 5) + (lane & 15));
+  uint4 pa[AMF][KKW], pb[2][KKW], qa[AMF][KKW], qb[2][KKW];
+  // Lane 32*h + r reads slot 16*COLS*(r >> 4) + 16*(2*kk + h) + (r & 15) of a fragment.
+  const uint8_t* lane_a = (const uint8_t*)ring +
+                          16 * (A_SLICE * wave + 16 * COLS * ((lane & 31) >> 4) + 16 * (lane >> 5) + (lane & 15));
+  const uint8_t* lane_b = lane_a + 16 * (A_PIECES + (B_SLICE - A_SLICE) * wave);
+  // Read number u of a step, in the order the next step consumes them: per K-step the rhs fragments, then the lhs.
+  auto read_unit = [&](int u, const uint8_t* stage, uint4 (*fa)[KKW], uint4 (*fb)[KKW]) {
+    const int kk = u / (AMF + 2), e = u % (AMF + 2);
+    if (e < 2) fb[e][kk] = *(const uint4*)(stage + (lane_b - (const uint8_t*)ring) + (FRAG_SLOTS * e + 32 * kk) * 16);
+    else fa[e - 2][kk] = *(const uint4*)(stage + (lane_a - (const uint8_t*)ring) + (FRAG_SLOTS * (e - 2) + 32 * kk) * 16);
+  };
 
   const uint8_t* load_a = lhs_base + min(AHEAD, last_chunk) * lhs_chunk_bytes;
   const uint8_t* load_b = rhs_base + min(AHEAD, last_chunk) * rhs_chunk_bytes;
@@ -1139,10 +1174,10 @@ void mmt4d_mfma_split_k_kernel(const MfmaArgs a) {
   uint32_t read_stage_off = STAGE_BYTES;
 
   // One step, as in the kernel above: two MFMAs ahead of the wait and the barrier, then the loads of the chunk
-  // three ahead and the LDS reads of the next chunk dealt out over four MFMAs, two MFMAs without memory work.
-  auto step = [&](const uint4 (*cur_a)[2], const uint4 (*cur_b)[2], uint4 (*nxt_a)[2], uint4 (*nxt_b)[2]) {
+  // AHEAD ahead and the LDS reads of the next chunk dealt out over four MFMAs, two MFMAs without memory work.
+  auto step = [&](const uint4 (*cur_a)[KKW], const uint4 (*cur_b)[KKW], uint4 (*nxt_a)[KKW], uint4 (*nxt_b)[KKW]) {
     auto multiply = [&](int m) {
-      const int kk = m >> 2, i = (m >> 1) & 1, j = m & 1;
+      const int kk = m / (AMF * 2), i = (m % (AMF * 2)) >> 1, j = m & 1;
       acc[i][j] = mfma<KIND>(cur_b[j][kk], cur_a[i][kk], acc[i][j]);
     };
     multiply(0);
@@ -1150,24 +1185,16 @@ void mmt4d_mfma_split_k_kernel(const MfmaArgs a) {
     __builtin_amdgcn_sched_barrier(0);
     wait_loads_but<LOADS*(AHEAD - 2)>();
     __builtin_amdgcn_s_barrier();
-    const uint8_t* read_a = lane_bytes + read_stage_off;
-    const uint8_t* read_b = read_a + OPERAND_PIECES * 16;
+    const uint8_t* stage = (const uint8_t*)ring + read_stage_off;
 #pragma unroll
     for (int m = 2; m < 8; ++m) {
       const int slot = m - 2;
       if (slot < 4) {
-        issue_load(2 * slot, load_stage_off, load_a, load_b);
-        issue_load(2 * slot + 1, load_stage_off, load_a, load_b);
+#pragma unroll
+        for (int n = slot * LOADS / 4; n < (slot + 1) * LOADS / 4; ++n) issue_load(n, load_stage_off, load_a, load_b);
         __builtin_amdgcn_sched_barrier(0);
-        // Read order: K-step 0 (rhs, lhs), then K-step 1: what the next step consumes first comes first.
-        const int kk = slot >> 1;
-        if ((slot & 1) == 0) {
-          nxt_b[0][kk] = *(const uint4*)(read_b + (32 * kk) * 16);
-          nxt_b[1][kk] = *(const uint4*)(read_b + (128 + 32 * kk) * 16);
-        } else {
-          nxt_a[0][kk] = *(const uint4*)(read_a + (32 * kk) * 16);
-          nxt_a[1][kk] = *(const uint4*)(read_a + (128 + 32 * kk) * 16);
-        }
+#pragma unroll
+        for (int u = slot * READS / 4; u < (slot + 1) * READS / 4; ++u) read_unit(u, stage, nxt_a, nxt_b);
       }
       multiply(m);
       if (m == 7) {
@@ -1192,12 +1219,7 @@ void mmt4d_mfma_split_k_kernel(const MfmaArgs a) {
   wait_loads_but<(AHEAD - 1) * LOADS>();
   __syncthreads();
 #pragma unroll
-  for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-    for (int f = 0; f < 2; ++f) {
-      pb[f][kk] = *(const uint4*)(lane_bytes + (OPERAND_PIECES + 128 * f + 32 * kk) * 16);
-      pa[f][kk] = *(const uint4*)(lane_bytes + (128 * f + 32 * kk) * 16);
-    }
+  for (int u = 0; u < READS; ++u) read_unit(u, (const uint8_t*)ring, pa, pb);
   int kc = 0;
   for (; kc + 1 < chunks; kc += 2) {
     step(pa, pb, qa, qb);
@@ -1207,24 +1229,32 @@ void mmt4d_mfma_split_k_kernel(const MfmaArgs a) {
   wait_loads_but<0>();
   __syncthreads();  // nobody reads operands from the ring any more
 
-  // The four partial tiles, summed in wavefront order. Quadrant q = 2*i + j of the tile ends up with wavefront q;
-  // partial[(q*4 + w)*16 + v][lane] is accumulator register v of wavefront w's fragment (i, j).
+  // The four partial tiles, summed in wavefront order. Wavefront w ends up with the fragments
+  // (OWN*(w >> 1) + o, w & 1), o < OWN: a block of (32*OWN) x 32 outputs. partial[((f*4 + w)*16 + v)][lane] is
+  // accumulator register v of wavefront w's fragment f = 2*i + j.
+  constexpr int OWN = AMF / 2;
   uint32_t* partial = (uint32_t*)ring;
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    if (q != wave) {
+  for (int f = 0; f < 2 * AMF; ++f) {
+    const int i = f >> 1, j = f & 1;
+    if (2 * (i / OWN) + j != wave) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const typename AccType<KIND>::scalar value = acc[q >> 1][q & 1][v];
-        partial[((q * 4 + wave) * 16 + v) * 64 + lane] = value_bits(value);
+        const typename AccType<KIND>::scalar value = acc[i][j][v];
+        partial[((f * 4 + wave) * 16 + v) * 64 + lane] = value_bits(value);
       }
     }
   }
   __syncthreads();
-  acc_t total[1][1];
-  {
-    // (selected without indexing the accumulator array by a run-time value)
-    const acc_t own = wave == 0 ? acc[0][0] : (wave == 1 ? acc[0][1] : (wave == 2 ? acc[1][0] : acc[1][1]));
+  acc_t total[OWN][1];
+#pragma unroll
+  for (int o = 0; o < OWN; ++o) {
+    // (the wavefront's own partial, selected without indexing the accumulator array by a run-time value)
+    acc_t own = acc[o][0];
+#pragma unroll
+    for (int w = 1; w < 4; ++w)
+      if (wave == w) own = acc[OWN * (w >> 1) + o][w & 1];
+    const int f = 2 * (OWN * (wave >> 1) + o) + (wave & 1);
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
       acc_t part;
@@ -1234,14 +1264,14 @@ void mmt4d_mfma_split_k_kernel(const MfmaArgs a) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           typename AccType<KIND>::scalar value;
-          set_from_bits(value, partial[((wave * 4 + w) * 16 + v) * 64 + lane]);
+          set_from_bits(value, partial[((f * 4 + w) * 16 + v) * 64 + lane]);
           part[v] = value;
         }
       }
-      if (w == 0) total[0][0] = part; else total[0][0] += part;
+      if (w == 0) total[o][0] = part; else total[o][0] += part;
     }
   }
-  store_block<KIND, false, NARROW, 1, 1>(a, total, first_row + 32 * (wave >> 1), first_col + 32 * (wave & 1), lane);
+  store_block<KIND, false, NARROW, OWN, 1>(a, total, first_row + 32 * OWN * (wave >> 1), first_col + 32 * (wave & 1), lane);
 }
 
 // Whether the direct-to-LDS kernel covers the problem: every lane can load 16
@@ -1287,19 +1317,24 @@ hipError_t launch_direct(MfmaArgs m, hipStream_t stream) {
   return hipGetLastError();
 }
 
-// The 64x64 tile with K split over the wavefronts: few block tiles, a long K that is whole steps of 256 bytes.
-inline bool split_k_pays(const MfmaArgs& m) {
+// The tiles with K split over the wavefronts. Returns the number of 32-row lhs fragments of the tile to use (2:
+// few 64x64 tiles and a long K; 4: at most 128 lhs rows, one row of 128x64 tiles), or 0 for the ordinary kernels.
+inline int split_k_tile(const MfmaArgs& m) {
   const int64_t rows = (int64_t)m.M << m.log2_M0, cols = (int64_t)m.N << m.log2_N0;
   const int64_t row_bytes = (int64_t)m.K * m.lhs_rb;
-  return ((rows + 63) / 64) * ((cols + 63) / 64) <= 128 && row_bytes % 256 == 0 && row_bytes >= 4096;
+  if (((rows + 63) / 64) * ((cols + 63) / 64) <= 128 && row_bytes % 256 == 0 && row_bytes >= 4096) return 2;
+  // (128 x 14336 x K: 8 KiB per row 27 -> 25 us, 96 rows 27 -> 23 us; at 4 KiB per row the prologue and the
+  // summing of the partial tiles cost what the steps gain: 18 -> 20 us.)
+  if (rows > 64 && rows <= 128 && row_bytes % 128 == 0 && row_bytes >= 8192) return 4;
+  return 0;
 }
 
-template <int KIND, bool NARROW>
+template <int KIND, bool NARROW, int AMF>
 hipError_t launch_split_k(MfmaArgs m, hipStream_t stream) {
   unsigned grid;
-  set_tile_grid(&m, 64, 64, &grid);
-  constexpr int lds_bytes = 4 * 2 * 64 * 256;
-  auto kernel = mmt4d_mfma_split_k_kernel<KIND, NARROW>;
+  set_tile_grid(&m, 32 * AMF, 64, &grid);
+  constexpr int lds_bytes = AMF == 2 ? 4 * 32768 : 6 * 24576;
+  auto kernel = mmt4d_mfma_split_k_kernel<KIND, NARROW, AMF>;
   const hipError_t attr = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
   if (attr != hipSuccess) return attr;
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds_bytes, stream, m);
@@ -1374,9 +1409,14 @@ template <int KIND, bool RHS_I4, int G, bool NARROW>
 hipError_t launch_variant(const MfmaArgs& m, hipStream_t stream, const char** name) {
   const bool direct = direct_covers<RHS_I4, G>(m);
   if constexpr (G == 16 && !RHS_I4 && KIND != kF32) {
-    if (direct && split_k_pays(m)) {
+    const int split = direct ? split_k_tile(m) : 0;
+    if (split == 2) {
       *name = "mmt4d_mfma_64x64_split_k";
-      return launch_split_k<KIND, NARROW>(m, stream);
+      return launch_split_k<KIND, NARROW, 2>(m, stream);
+    }
+    if (split == 4) {
+      *name = "mmt4d_mfma_128x64_split_k";
+      return launch_split_k<KIND, NARROW, 4>(m, stream);
     }
   }
   const TileChoice* tile;

@@ -258,7 +258,25 @@ def test_split_k_tile(gpu_lib, flags, M0, N0, K0):
     run_case(gpu_lib, flags, max(1, 16 // M0), 48 // N0, 41 * per_step, M0, N0, K0, name, accumulate=True, seed=3)
     # K not whole steps of 256 bytes, or too short to matter: the ordinary 64x64 tile
     run_case(gpu_lib, flags, 72 // M0 + 1, 88 // N0, 16 * per_step + 64 // (K0 * e), M0, N0, K0, "mmt4d_mfma_64x64", seed=4)
-    run_case(gpu_lib, flags, 72 // M0 + 1, 88 // N0, 8 * per_step, M0, N0, K0, "mmt4d_mfma_64x64", seed=5)
+    run_case(gpu_lib, flags, max(1, 48 // M0), 88 // N0, 8 * per_step, M0, N0, K0, "mmt4d_mfma_64x64", seed=5)
+
+
+# The same with one row of 128x64 tiles (65 .. 128 lhs rows against many rhs rows): 128 bytes of K per row and step.
+@pytest.mark.parametrize("flags,M0,N0,K0", [(abi.MMT4D_TYPE_S8S8S32, 16, 16, 64), (abi.MMT4D_TYPE_S8S8S32, 8, 8, 16),
+                                            (abi.MMT4D_TYPE_F16F16F32, 16, 16, 16), (abi.MMT4D_TYPE_BF16BF16F32, 16, 16, 8),
+                                            (abi.MMT4D_TYPE_BF16BF16F32, 4, 16, 8), (abi.MMT4D_TYPE_F16F16F16, 16, 16, 8)])
+def test_split_k_tile_128_rows(gpu_lib, flags, M0, N0, K0):
+    e = 1 if flags == abi.MMT4D_TYPE_S8S8S32 else 2
+    per_step = max(1, 128 // (K0 * e))              # k steps per 128 bytes of a row
+    name = "mmt4d_mfma_128x64_split_k"
+    cols = 9000 // N0
+    run_case(gpu_lib, flags, 128 // M0, cols, 64 * per_step, M0, N0, K0, name, accumulate=True, out_pad=8, seed=1)
+    run_case(gpu_lib, flags, 100 // M0, cols + 3, 65 * per_step, M0, N0, K0, name, lhs_pad=64 // e, rhs_pad=32 // e,
+             offsets=(16 // e, 48 // e, 4), seed=2)
+    run_case(gpu_lib, flags, 80 // M0, cols, 97 * per_step, M0, N0, K0, name, accumulate=True, seed=3)
+    # 64 rows or fewer, or a K too short to pay for summing the partial tiles: the ordinary tiles
+    run_case(gpu_lib, flags, 64 // M0, cols, 64 * per_step, M0, N0, K0, "mmt4d_mfma_64x64", seed=4)
+    run_case(gpu_lib, flags, 128 // M0, cols, 32 * per_step, M0, N0, K0, "mmt4d_mfma_128x64", seed=5)
 
 
 def test_ragged_K_on_the_register_staged_kernel(gpu_lib):
