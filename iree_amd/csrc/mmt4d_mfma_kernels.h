@@ -1319,13 +1319,15 @@ hipError_t launch_direct(MfmaArgs m, hipStream_t stream) {
 
 // The tiles with K split over the wavefronts. Returns the number of 32-row lhs fragments of the tile to use (2:
 // few 64x64 tiles and a long K; 4: at most 128 lhs rows, one row of 128x64 tiles), or 0 for the ordinary kernels.
-inline int split_k_tile(const MfmaArgs& m) {
+inline int split_k_tile(const MfmaArgs& m, bool int8) {
   const int64_t rows = (int64_t)m.M << m.log2_M0, cols = (int64_t)m.N << m.log2_N0;
   const int64_t row_bytes = (int64_t)m.K * m.lhs_rb;
   if (((rows + 63) / 64) * ((cols + 63) / 64) <= 128 && row_bytes % 256 == 0 && row_bytes >= 4096) return 2;
-  // (128 x 14336 x K: 8 KiB per row 27 -> 25 us, 96 rows 27 -> 23 us; at 4 KiB per row the prologue and the
-  // summing of the partial tiles cost what the steps gain: 18 -> 20 us.)
-  if (rows > 64 && rows <= 128 && row_bytes % 128 == 0 && row_bytes >= 8192) return 4;
+  // (bf16 128 x 14336 x 4096 27 -> 25 us, 96 rows 27 -> 23 us, 128 x 8192 x 8192 40 -> 36 us. Not with less K per
+  // row, where the prologue and the summing of the partial tiles cost what the steps gain; not for int8, which does
+  // twice the MFMA work per byte: 128 x 14336 x 8192 29 -> 31 us; not with more tiles than compute units, where
+  // 128x128 tiles win: bf16 128 x 28672 x 4096 41 -> 49 us.)
+  if (!int8 && rows > 64 && rows <= 128 && cols <= 256 * 64 && row_bytes % 128 == 0 && row_bytes >= 8192) return 4;
   return 0;
 }
 
@@ -1409,7 +1411,7 @@ template <int KIND, bool RHS_I4, int G, bool NARROW>
 hipError_t launch_variant(const MfmaArgs& m, hipStream_t stream, const char** name) {
   const bool direct = direct_covers<RHS_I4, G>(m);
   if constexpr (G == 16 && !RHS_I4 && KIND != kF32) {
-    const int split = direct ? split_k_tile(m) : 0;
+    const int split = direct ? split_k_tile(m, KIND == kI8) : 0;
     if (split == 2) {
       *name = "mmt4d_mfma_64x64_split_k";
       return launch_split_k<KIND, NARROW, 2>(m, stream);

@@ -261,12 +261,13 @@ def test_split_k_tile(gpu_lib, flags, M0, N0, K0):
     run_case(gpu_lib, flags, max(1, 48 // M0), 88 // N0, 8 * per_step, M0, N0, K0, "mmt4d_mfma_64x64", seed=5)
 
 
-# The same with one row of 128x64 tiles (65 .. 128 lhs rows against many rhs rows): 128 bytes of K per row and step.
-@pytest.mark.parametrize("flags,M0,N0,K0", [(abi.MMT4D_TYPE_S8S8S32, 16, 16, 64), (abi.MMT4D_TYPE_S8S8S32, 8, 8, 16),
-                                            (abi.MMT4D_TYPE_F16F16F32, 16, 16, 16), (abi.MMT4D_TYPE_BF16BF16F32, 16, 16, 8),
-                                            (abi.MMT4D_TYPE_BF16BF16F32, 4, 16, 8), (abi.MMT4D_TYPE_F16F16F16, 16, 16, 8)])
+# The same with one row of 128x64 tiles (65 .. 128 lhs rows against many rhs rows, f16 / bf16): 128 bytes of K per row
+# and step.
+@pytest.mark.parametrize("flags,M0,N0,K0", [(abi.MMT4D_TYPE_F16F16F32, 16, 16, 16), (abi.MMT4D_TYPE_BF16BF16F32, 16, 16, 8),
+                                            (abi.MMT4D_TYPE_BF16BF16F32, 4, 16, 8), (abi.MMT4D_TYPE_F16F16F16, 16, 16, 8),
+                                            (abi.MMT4D_TYPE_BF16BF16BF16, 8, 8, 32), (abi.MMT4D_TYPE_F16F16F32, 2, 4, 16)])
 def test_split_k_tile_128_rows(gpu_lib, flags, M0, N0, K0):
-    e = 1 if flags == abi.MMT4D_TYPE_S8S8S32 else 2
+    e = 2
     per_step = max(1, 128 // (K0 * e))              # k steps per 128 bytes of a row
     name = "mmt4d_mfma_128x64_split_k"
     cols = 9000 // N0
