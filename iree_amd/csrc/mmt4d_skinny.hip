@@ -11,8 +11,8 @@
 // k step at all. Here nothing is transposed. The rhs of one tile row
 // (N0 rows x K k steps, one contiguous stream) is read 16 bytes per lane, and
 // each lane multiplies the 16 / G rows it holds with the lhs pieces of its
-// k step on the VALU (v_dot4_i32_i8, v_dot2_f32_f16, FMAs), keeping one
-// accumulator per (lhs row, rhs row). The lhs is small and comes through the
+// k step on the VALU (v_dot4_i32_i8, v_dot2_i32_i16, FMAs on 16-bit floats
+// widened to f32), keeping one accumulator per (lhs row, rhs row). The lhs is small and comes through the
 // caches. At the end the lanes that hold the same rhs rows (they differ in
 // k step) are summed with a butterfly of lane exchanges, the wavefronts of the
 // workgroup (which split the stream between them) through LDS, both in a
@@ -52,7 +52,7 @@ struct SkinnyArgs {
   uint8_t* out;
   int64_t lhs_stride_bytes, rhs_stride_bytes;
   int64_t out_stride0;  // elements
-  int64_t tile_bytes;   // K * N0 * G: one rhs tile row
+  int64_t tile_bytes;   // K * N0 * (bytes of an rhs row piece): one rhs tile row
   int32_t rows;         // M * M0
   int32_t N, K;
   int32_t log2_M0, log2_N0;
@@ -64,11 +64,11 @@ template <> struct Acc<kI8> { typedef int32_t type; };
 template <> struct Acc<kI16> { typedef int32_t type; };
 template <> struct Acc<kI16U4> { typedef int32_t type; };
 template <> struct Acc<kI8I4> { typedef int32_t type; };
-// The lhs piece of one k step in registers: G bytes, zero-extended to two
-// dwords; 16 bytes (8 values of 16 bits) against 8 nibbles of the rhs.
+// The lhs piece of one k step in registers. Same bytes as an rhs piece (G, zero-extended to two dwords), except:
+// s16u4s32: 8 values of 16 bits against 8 nibbles; s8s4s32: 8 or 16 bytes against as many nibbles, kept as one
+// dword of the even and one of the odd bytes per 8.
 template <int KIND> struct LhsPiece { typedef uint2 type; };
 template <> struct LhsPiece<kI16U4> { typedef uint4 type; };
-// int4 rhs: per 8 lhs bytes one dword of the even and one of the odd ones.
 template <> struct LhsPiece<kI8I4> { typedef uint4 type; };
 
 __device__ __forceinline__ int32_t dot2_i16(uint32_t a, uint32_t b, int32_t c) {
