@@ -179,8 +179,25 @@ def test_mmt4d_info_reports_specialised_kernels():
                             (abi.MMT4D_TYPE_S8S4S32, 16, 16, 32), (abi.MMT4D_TYPE_BF16BF16F32, 1, 16, 8),
                             (abi.MMT4D_TYPE_BF16BF16F32, 4, 16, 8), (abi.MMT4D_TYPE_BF16BF16F32, 16, 16, 8)]:
         assert lib.iree_uk_mmt4d_info(m0, n0, k0, t, None) == 1, (t, m0, n0, k0)
+    # The tile shapes the reference's x86-64 and Arm targets compile in (mmt4d_x86_64_tiles.inl,
+    # mmt4d_arm_64_tiles.inl), wide and narrow; 16-bit outputs with the roundings between k steps skipped.
+    skip = abi.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS
+    for (t, m0, n0, k0) in [(abi.MMT4D_TYPE_S8S8S32, 16, 16, 2), (abi.MMT4D_TYPE_S8S8S32, 1, 16, 2),
+                            (abi.MMT4D_TYPE_S8S8S32, 4, 8, 2), (abi.MMT4D_TYPE_F16F16F32, 16, 16, 1),
+                            (abi.MMT4D_TYPE_F16F16F32, 1, 8, 1), (abi.MMT4D_TYPE_F16F16F16 | skip, 16, 16, 1),
+                            (abi.MMT4D_TYPE_BF16BF16F32, 2, 16, 2), (abi.MMT4D_TYPE_BF16BF16BF16 | skip, 8, 8, 4),
+                            (abi.MMT4D_TYPE_F32F32F32, 1, 16, 1), (abi.MMT4D_TYPE_F32F32F32, 16, 16, 1),
+                            (abi.MMT4D_TYPE_S8S8S32, 8, 8, 8), (abi.MMT4D_TYPE_S8S8S32, 2, 8, 4),
+                            (abi.MMT4D_TYPE_S16S16S32, 1, 16, 2), (abi.MMT4D_TYPE_S16U4S32, 1, 32, 8),
+                            (abi.MMT4D_TYPE_S8S4S32, 4, 8, 8), (abi.MMT4D_TYPE_S8S4S32, 1, 8, 16)]:
+        assert lib.iree_uk_mmt4d_info(m0, n0, k0, t, None) == 1, (hex(t), m0, n0, k0)
     assert lib.iree_uk_mmt4d_info(9, 6, 3, abi.MMT4D_TYPE_S8S8S32, None) == 0
     assert lib.iree_uk_mmt4d_info(8, 8, 4, 0x0B, None) == 0
+    # What only the generic kernel takes: one-byte row pieces, 16-bit integers in 16-row tiles, f16f16f16 with a
+    # rounding after every k step.
+    assert lib.iree_uk_mmt4d_info(8, 8, 1, abi.MMT4D_TYPE_S8S8S32, None) == 0
+    assert lib.iree_uk_mmt4d_info(16, 16, 2, abi.MMT4D_TYPE_S16S16S32, None) == 0
+    assert lib.iree_uk_mmt4d_info(16, 16, 1, abi.MMT4D_TYPE_F16F16F16, None) == 0
 
 
 def test_query_tile_sizes_roles_are_consistent():
