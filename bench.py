@@ -190,6 +190,14 @@ def _also(torch, lib, abi, synth, steps, warmup):
         "kernel": lib.iree_uk_mi355x_last_kernel().decode(), "ms": round(ms, 5),
         "value": round(2.0 * 4096 ** 3 / ms / 1e9, 1), "unit": "TOP/s",
         "frac_of_peak": round(2.0 * 4096 ** 3 / ms / 1e9 / PEAK_INT8_TOPS, 4)}
+    # The same product as a 32 x 32 grid of 128x128 tiles (4 x 4 intrinsics per subgroup, 2 x 2 subgroups): several
+    # workgroups per compute unit.
+    ms, _ = _time_launches(torch, lambda: lib.iree_uk_mi355x_multi_mma_i32_16x16x64_i8(
+        ta.data_ptr(), tb.data_ptr(), tc.data_ptr(), 32, 32, 64, 4, 2, 4, 2, 1), steps, warmup)
+    res["multi_mma_i32_16x16x64_i8_4096_device_ukernel_128x128_tiles"] = {
+        "kernel": lib.iree_uk_mi355x_last_kernel().decode(), "ms": round(ms, 5),
+        "value": round(2.0 * 4096 ** 3 / ms / 1e9, 1), "unit": "TOP/s",
+        "frac_of_peak": round(2.0 * 4096 ** 3 / ms / 1e9 / PEAK_INT8_TOPS, 4)}
     del ta, tb, tc
     # s8s4s32 512 x 11008 x 4096, tiles 16x16x32.
     lhs = torch.from_numpy(synth.uniform_int8(5, 0, 512 * 4096)).cuda()

@@ -22,8 +22,7 @@ struct MultiMmaArgs {
 template <int IM, int SM, int IN, int SN, int IK>
 __global__ __launch_bounds__(64 * SM * SN) void multi_mma_kernel(const MultiMmaArgs g) {
   extern __shared__ __attribute__((aligned(16))) int8_t workgroup_memory[];
-  constexpr int32_t shared_bytes =
-      2 * 16 * ((SN > 1 ? 64 * IM * IK * SM : 0) + (SM > 1 ? 64 * IN * IK * SN : 0));
+  constexpr int32_t shared_bytes = iree_uk_amdgpu::shared_memory_bytes_for(IM, SM, IN, SN, IK);
   const int64_t outer_m = blockIdx.y, outer_n = blockIdx.x;
   const int tid = threadIdx.x, lane = tid % 64, subgroup = tid / 64;
   const int subgroup_n = subgroup % SN, subgroup_m = subgroup / SN;
