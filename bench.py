@@ -138,6 +138,17 @@ def _also(torch, lib, abi, synth, steps, warmup):
     mm("mmt4d_f16f16f32_4096_16x16x16_acc", abi.MMT4D_TYPE_F16F16F32, 256, 256, 256, 16, 16, 16,
        f16_operand(3, 0, n, 1.0 / 64), f16_operand(3, 1, n, 1.0 / 64), torch.float32,
        PEAK_F16_TFLOPS, "TFLOP/s", acc=True)
+    # 4096^3 in the tile shapes an x86-64 caller passes (mmt4d_x86_64_tiles.inl): 2-byte row pieces for int8 with
+    # VNNI and for f16, 4-byte for bf16; operands of the same distributions as above.
+    xl, xr = torch.from_numpy(synth.uniform_int8(0, 0, n)).cuda(), torch.from_numpy(synth.uniform_int8(0, 1, n)).cuda()
+    mm("mmt4d_s8s8s32_4096_x86_tile_16x16x2", abi.MMT4D_TYPE_S8S8S32, 256, 256, 2048, 16, 16, 2, xl, xr, torch.int32,
+       PEAK_INT8_TOPS, "TOP/s")
+    del xl, xr
+    mm("mmt4d_f16f16f32_4096_x86_tile_16x16x1", abi.MMT4D_TYPE_F16F16F32, 256, 256, 4096, 16, 16, 1,
+       f16_operand(3, 0, n, 1.0 / 64), f16_operand(3, 1, n, 1.0 / 64), torch.float32, PEAK_F16_TFLOPS, "TFLOP/s")
+    mm("mmt4d_bf16bf16f32_4096_x86_tile_16x16x2", abi.MMT4D_TYPE_BF16BF16F32, 256, 256, 2048, 16, 16, 2,
+       f16_operand(4, 0, n, 1.0, bf16=True), f16_operand(4, 10, n, 0.02, bf16=True), torch.float32, PEAK_F16_TFLOPS,
+       "TFLOP/s")
     # The headline problem once more with all-zero operands: same kernel, same
     # instruction stream, same memory traffic. The part sustains a higher clock
     # when the data does not toggle, which is what the difference to the headline
