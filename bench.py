@@ -158,7 +158,7 @@ def _also(torch, lib, abi, synth, steps, warmup):
        zl, zl, torch.int32, PEAK_INT8_TOPS, "TOP/s")
     del zl
     # What the matrix pipe sustains on this device, measured by the
-    # library's probe: the 256x256 kernel's inner-loop instruction mix with no
+    # benchmark's probe (a helper library of its own): the 256x256 kernel's inner-loop instruction mix with no
     # HBM traffic, no prologue and no epilogue, on all-zero bytes, on the
     # headline's uniformly random int8 and on the f16 / bf16 configurations'
     # operands, without and with the loop's LDS reads, loads to LDS and barrier.
@@ -176,7 +176,7 @@ def _also(torch, lib, abi, synth, steps, warmup):
             (abi.MMT4D_TYPE_BF16BF16F32, PEAK_F16_TFLOPS, "TFLOP/s", "bf16_normal_sigma_0.02", bf16)):
         for traffic in (0, 1):
             tops, mhz = C.c_double(), C.c_double()
-            rc = lib.iree_uk_mi355x_probe_matrix_pipe(type_flag, buf.data_ptr(), buf.numel() * buf.element_size(),
+            rc = library.load_bench_probe().uk_bench_probe_matrix_pipe(type_flag, buf.data_ptr(), buf.numel() * buf.element_size(),
                                                       traffic, 4096, C.byref(tops), C.byref(mhz))
             if rc != 0:
                 raise RuntimeError("matrix pipe probe failed: HIP error %d" % rc)

@@ -249,26 +249,6 @@ int iree_uk_mi355x_multi_mma_i32_16x16x64_i8(const void* a, const void* b, void*
                                              int32_t subgroups_m, int32_t intrinsics_n, int32_t subgroups_n,
                                              int32_t intrinsics_k);
 
-/* A measuring stick with no counterpart in the reference: the rate the matrix
- * pipe of the current device sustains on the given operand bytes, for the
- * operand type of `mmt4d_type` (IREE_UK_FLAG_MMT4D_TYPE_S8S8S32, _F16F16F32 or
- * _BF16BF16F32). One workgroup per compute unit runs the instruction mix of
- * the 256x256 mmt4d kernel's inner loop for `steps` steps (even, >= 2; 32
- * MFMAs per wavefront and step: 32x32x32 int8 or 32x32x16 f16/bf16), with
- * operands taken from `operand_bytes` (device memory, at least 2 MiB are
- * used): without memory instructions (memory_traffic == 0), or with each
- * step's LDS reads, loads to LDS (cache hits) and barrier. Writes the rate in
- * 1e12 op/s and the shader clock observed (cycle counter of one workgroup over
- * the launch's duration, MHz); either pointer may be NULL. The device's
- * sustained clock depends on how many operand bits toggle, so all-zero and
- * random bytes give different rates at the same cycle count; the result bounds
- * what any kernel built on these instructions reaches on such data. Allocates
- * a few bytes of device memory for the call, synchronises the device's null
- * stream. Returns 0 or a HIP error code. */
-int iree_uk_mi355x_probe_matrix_pipe(uint32_t mmt4d_type, const void* operand_bytes, long long operand_size,
-                                     int memory_traffic, int steps, double* tera_ops_per_second,
-                                     double* shader_mhz);
-
 /* Library version, MAJOR*10000 + MINOR*100 + PATCH. */
 int iree_uk_mi355x_version(void);
 

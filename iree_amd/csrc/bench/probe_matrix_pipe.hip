@@ -1,4 +1,5 @@
-// A measuring stick, not part of the matmul path: what the matrix pipe of the
+// A measuring stick for the benchmark, built into its own helper library
+// (libuk_bench_probe.so), not into the microkernel library: what the matrix pipe of the
 // device sustains on given operand bytes, for int8, f16 or bf16 operands. One
 // workgroup of four wavefronts per compute unit runs the inner loop of the
 // 256x256 mmt4d kernel stripped to its instruction mix: per step 32
@@ -125,7 +126,7 @@ void probe_kernel(const uint8_t* src, int32_t* sink, int steps, long long* cycle
 
 }  // namespace
 
-UK_API int iree_uk_mi355x_probe_matrix_pipe(uint32_t mmt4d_type, const void* operand_bytes, long long operand_size,
+UK_API int uk_bench_probe_matrix_pipe(uint32_t mmt4d_type, const void* operand_bytes, long long operand_size,
                                             int memory_traffic, int steps, double* tera_ops_per_second,
                                             double* shader_mhz) {
   if (operand_bytes == nullptr || operand_size < kOperandBytesNeeded || steps < 2 || (steps & 1)) {

@@ -66,6 +66,14 @@ void report_failure(const char* file, int line, const char* function, const char
     }                                                                         \
   } while (0)
 
+// outer * tile >= size for non-negative values, without forming a product
+// that may not fit.
+bool tiles_cover(int64_t outer, int64_t tile, int64_t size) {
+  if (size == 0) return true;
+  if (outer == 0 || tile == 0) return false;
+  return outer >= size / tile + (size % tile != 0);
+}
+
 bool in_unsigned_range(int64_t v, int bits) { return v >= 0 && v < ((int64_t)1 << bits); }
 
 // True if a kernel on the current device may dereference `p`.
@@ -80,14 +88,24 @@ bool device_accessible(const void* p) {
          attr.type == hipMemoryTypeHost;
 }
 
-// Per-thread device staging buffers for host operands (grow-only).
+// Per-thread device staging buffers for host operands (grow-only, released
+// when the thread exits).
 struct StageBuffer {
   void* ptr = nullptr;
   size_t capacity = 0;
+  ~StageBuffer() {
+    // At process teardown the HIP runtime may already be gone: errors are moot.
+    if (ptr) (void)hipFree(ptr);
+  }
 };
 thread_local StageBuffer tl_stage[3];
 
-bool stage_reserve(int slot, size_t bytes, void** out) {
+// Where the calling entry point mirrors host operands.
+struct Stager {
+};
+
+bool stage_reserve(Stager& stager, int slot, size_t bytes, void** out) {
+  (void)stager;
   StageBuffer& s = tl_stage[slot];
   if (s.capacity < bytes) {
     if (s.ptr) UK_HIP_OK(hipFree(s.ptr));
@@ -101,18 +119,56 @@ bool stage_reserve(int slot, size_t bytes, void** out) {
   return true;
 }
 
-// A strided set of rows inside one operand: `rows` rows of `width` bytes,
-// `pitch` bytes apart. span() is the byte count from the first to the last
-// touched byte.
-struct RowRegion {
-  int64_t rows, width, pitch;
-  int64_t span() const { return rows <= 0 || width <= 0 ? 0 : (rows - 1) * pitch + width; }
+// int64 arithmetic on caller-provided sizes that records overflow instead of
+// wrapping (the checks of the reference admit sizes whose products do not fit).
+struct Checked {
+  bool ok = true;
+  int64_t mul(int64_t a, int64_t b) {
+    int64_t r = 0;
+    if (__builtin_mul_overflow(a, b, &r)) ok = false;
+    return ok ? r : 0;
+  }
+  int64_t add(int64_t a, int64_t b) {
+    int64_t r = 0;
+    if (__builtin_add_overflow(a, b, &r)) ok = false;
+    return ok ? r : 0;
+  }
+  // Bytes of `elems` elements of `bits` bits each (sub-byte types: the callers
+  // have checked that the count is a whole number of bytes).
+  int64_t bytes(int64_t elems, int bits) { return bits >= 8 ? mul(elems, bits / 8) : elems / (8 / bits); }
 };
 
+// `base + bytes` without the undefined behaviour of pointer arithmetic outside
+// an object: callers may pass `allocation - offset` as the base.
+const uint8_t* offset_pointer(const void* base, int64_t bytes) {
+  return (const uint8_t*)((uintptr_t)base + (uintptr_t)bytes);
+}
+
+// A strided set of rows inside one operand: `rows` rows of `width` bytes,
+// `pitch` bytes apart; `span` is the byte count from the first to the last
+// touched byte.
+struct RowRegion {
+  int64_t rows = 0, width = 0, pitch = 0, span = 0;
+};
+
+RowRegion make_region(Checked& c, int64_t rows, int64_t width, int64_t pitch) {
+  RowRegion r;
+  r.rows = rows; r.width = width; r.pitch = pitch;
+  r.span = rows <= 0 || width <= 0 ? 0 : c.add(c.mul(rows - 1, pitch), width);
+  return r;
+}
+
+// The same bytes as one row (for operands whose rows overlap or interleave).
+RowRegion as_one_span(const RowRegion& r) {
+  RowRegion o;
+  o.rows = 1; o.width = r.span; o.pitch = 0; o.span = r.span;
+  return o;
+}
+
 bool copy_rows(void* dst, const void* src, const RowRegion& r, hipMemcpyKind kind, hipStream_t s) {
-  if (r.span() == 0) return true;
+  if (r.span == 0) return true;
   if (r.rows == 1 || r.pitch == r.width) {
-    UK_HIP_OK(hipMemcpyAsync(dst, src, (size_t)r.span(), kind, s));
+    UK_HIP_OK(hipMemcpyAsync(dst, src, (size_t)r.span, kind, s));
   } else {
     UK_HIP_OK(hipMemcpy2DAsync(dst, (size_t)r.pitch, src, (size_t)r.pitch, (size_t)r.width,
                                (size_t)r.rows, kind, s));
@@ -128,12 +184,23 @@ struct Staged {
   void* dev = nullptr;
 };
 
-bool stage_operand(int slot, const void* ptr, const RowRegion& region, bool upload,
+bool stage_operand(Stager& stager, int slot, const void* ptr, const RowRegion& region, bool upload,
                    hipStream_t stream, Staged* st, const void** dev_ptr) {
   *dev_ptr = ptr;
-  if (tl_async || region.span() == 0 || device_accessible(ptr)) return true;
+  if (region.span == 0) return true;
+  const bool on_device = device_accessible(ptr);
+  if (tl_async) {
+    // Nothing is staged in asynchronous mode, and a host address must not
+    // reach a kernel: the device would fault.
+    if (!on_device) {
+      report_failure(__FILE__, __LINE__, __func__, "asynchronous mode needs device-accessible operands");
+      return false;
+    }
+    return true;
+  }
+  if (on_device) return true;
   void* d = nullptr;
-  if (!stage_reserve(slot, (size_t)region.span(), &d)) return false;
+  if (!stage_reserve(stager, slot, (size_t)region.span, &d)) return false;
   if (upload && !copy_rows(d, ptr, region, hipMemcpyHostToDevice, stream)) return false;
   st->host = ptr;
   st->dev = d;
@@ -194,7 +261,9 @@ int unpack_elem_bytes(uint32_t flags) {
 // mmt4d
 //===----------------------------------------------------------------------===//
 
-UK_API void iree_uk_mmt4d_p(const iree_uk_mmt4d_params_t* p) {
+namespace {
+
+void mmt4d_impl(const iree_uk_mmt4d_params_t* p, Stager& stager) {
   tl_last_kernel = "";
   UK_REQUIRE(p != nullptr);
   // Checks of mmt4d.c:12-48.
@@ -213,10 +282,11 @@ UK_API void iree_uk_mmt4d_p(const iree_uk_mmt4d_params_t* p) {
   UK_REQUIRE(ob >= 8);
   UK_REQUIRE((p->K0 * lb) % 8 == 0);
   UK_REQUIRE((p->K0 * rb) % 8 == 0);
-  UK_REQUIRE((p->lhs_stride0 * lb) % 8 == 0);
-  UK_REQUIRE((p->rhs_stride0 * rb) % 8 == 0);
-  UK_REQUIRE((p->lhs_offset * lb) % 8 == 0);
-  UK_REQUIRE((p->rhs_offset * rb) % 8 == 0);
+  // (stride * bits) % 8 without forming the product.
+  UK_REQUIRE(((p->lhs_stride0 % 8) * lb) % 8 == 0);
+  UK_REQUIRE(((p->rhs_stride0 % 8) * rb) % 8 == 0);
+  UK_REQUIRE(((p->lhs_offset % 8) * lb) % 8 == 0);
+  UK_REQUIRE(((p->rhs_offset % 8) * rb) % 8 == 0);
 
   // Early exits of mmt4d.c:105-113. (K == 0 without ACCUMULATE still has to
   // zero the output tiles, so it goes on to a kernel.)
@@ -224,24 +294,36 @@ UK_API void iree_uk_mmt4d_p(const iree_uk_mmt4d_params_t* p) {
   if (p->M == 0 || p->N == 0 || (p->K == 0 && accumulate)) return;
   if (p->M0 == 0 || p->N0 == 0) return;  // empty tiles: nothing to write
 
-  const RowRegion lhs_region{p->M, p->K * p->M0 * p->K0 * lb / 8, p->lhs_stride0 * lb / 8};
-  const RowRegion rhs_region{p->N, p->K * p->N0 * p->K0 * rb / 8, p->rhs_stride0 * rb / 8};
-  const RowRegion out_region{p->M, p->N * p->M0 * p->N0 * ob / 8, p->out_stride0 * ob / 8};
-  // Rows may not overlap (strides of a one-row operand are irrelevant).
-  UK_REQUIRE(p->M == 1 || lhs_region.pitch >= lhs_region.width);
-  UK_REQUIRE(p->N == 1 || rhs_region.pitch >= rhs_region.width);
+  Checked c;
+  const RowRegion lhs_region = make_region(c, p->M, c.bytes(c.mul(p->K, (int64_t)p->M0 * p->K0), lb),
+                                           c.bytes(p->lhs_stride0, lb));
+  const RowRegion rhs_region = make_region(c, p->N, c.bytes(c.mul(p->K, (int64_t)p->N0 * p->K0), rb),
+                                           c.bytes(p->rhs_stride0, rb));
+  const RowRegion out_region = make_region(c, p->M, c.bytes(c.mul(p->N, (int64_t)p->M0 * p->N0), ob),
+                                           c.bytes(p->out_stride0, ob));
+  const int64_t lhs_offset_bytes = c.bytes(p->lhs_offset, lb), rhs_offset_bytes = c.bytes(p->rhs_offset, rb),
+                out_offset_bytes = c.bytes(p->out_offset, ob);
+  UK_REQUIRE(c.ok && "operand extents fit int64");
+  // The reference puts no condition on the strides (mmt4d.c:12-48). Operand
+  // rows may overlap or coincide (stride 0 broadcasts one panel); they are
+  // only read. Rows of the output may not overlap here, because they are
+  // written concurrently, and strides that walk backwards are not supported.
+  UK_REQUIRE(p->M == 1 || p->lhs_stride0 >= 0);
+  UK_REQUIRE(p->N == 1 || p->rhs_stride0 >= 0);
   UK_REQUIRE(p->M == 1 || out_region.pitch >= out_region.width);
 
-  const void* lhs = (const uint8_t*)p->lhs_buffer + p->lhs_offset * lb / 8;
-  const void* rhs = (const uint8_t*)p->rhs_buffer + p->rhs_offset * rb / 8;
-  const void* out = (uint8_t*)p->out_buffer + p->out_offset * ob / 8;
+  const void* lhs = offset_pointer(p->lhs_buffer, lhs_offset_bytes);
+  const void* rhs = offset_pointer(p->rhs_buffer, rhs_offset_bytes);
+  const void* out = offset_pointer(p->out_buffer, out_offset_bytes);
 
   hipStream_t stream = tl_stream;
   Staged s_lhs, s_rhs, s_out;
   const void *d_lhs, *d_rhs, *d_out;
-  if (!stage_operand(0, lhs, lhs_region, true, stream, &s_lhs, &d_lhs)) return;
-  if (!stage_operand(1, rhs, rhs_region, true, stream, &s_rhs, &d_rhs)) return;
-  if (!stage_operand(2, out, out_region, accumulate, stream, &s_out, &d_out)) return;
+  // A host operand whose rows overlap is staged as one span.
+  auto as_copied = [](const RowRegion& r) { return r.rows > 1 && r.pitch < r.width ? as_one_span(r) : r; };
+  if (!stage_operand(stager, 0, lhs, as_copied(lhs_region), true, stream, &s_lhs, &d_lhs)) return;
+  if (!stage_operand(stager, 1, rhs, as_copied(rhs_region), true, stream, &s_rhs, &d_rhs)) return;
+  if (!stage_operand(stager, 2, out, out_region, accumulate, stream, &s_out, &d_out)) return;
 
   uk::Mmt4dArgs a;
   a.lhs = (const uint8_t*)d_lhs;
@@ -258,6 +340,13 @@ UK_API void iree_uk_mmt4d_p(const iree_uk_mmt4d_params_t* p) {
   if (!launcher) launcher = uk::launch_mmt4d_generic;
   if (!launch_ok(launcher(a, stream, &tl_last_kernel), "mmt4d")) return;
   finish(stream, s_out, out_region, s_lhs.host || s_rhs.host || s_out.host);
+}
+
+}  // namespace
+
+UK_API void iree_uk_mmt4d_p(const iree_uk_mmt4d_params_t* p) {
+  Stager stager;
+  mmt4d_impl(p, stager);
 }
 
 UK_API void iree_uk_mmt4d(const void* lhs_buffer, iree_uk_index_t lhs_offset,
@@ -319,26 +408,30 @@ UK_API void iree_uk_pack_p(const iree_uk_pack_params_t* p) {
   UK_REQUIRE(p->in_stride0 >= 0);
   UK_REQUIRE(p->in_stride1 >= 0);
   UK_REQUIRE(p->out_stride0 >= 0);
-  UK_REQUIRE(p->out_stride1 == p->out_size2 * p->out_size3);
+  Checked c;
+  UK_REQUIRE(p->out_stride1 == c.mul(p->out_size2, p->out_size3) && c.ok);
   int64_t outer0 = p->out_size0, outer1 = p->out_size1;
   int64_t tile0 = p->out_size2, tile1 = p->out_size3;
   if (p->flags & IREE_UK_FLAG_PACK_TRANSPOSE_OUTER) { int64_t t = outer0; outer0 = outer1; outer1 = t; }
   if (p->flags & IREE_UK_FLAG_PACK_TRANSPOSE_INNER) { int64_t t = tile0; tile0 = tile1; tile1 = t; }
-  UK_REQUIRE(outer0 * tile0 >= p->in_size0);
-  UK_REQUIRE(outer1 * tile1 >= p->in_size1);
+  UK_REQUIRE(tiles_cover(outer0, tile0, p->in_size0));
+  UK_REQUIRE(tiles_cover(outer1, tile1, p->in_size1));
 
   // Early exit of pack.c:106-109.
   if (p->out_size0 == 0 || p->out_size1 == 0 || p->out_size2 == 0 || p->out_size3 == 0) return;
 
   const bool have_input = p->in_size0 > 0 && p->in_size1 > 0;
-  const RowRegion in_region{have_input ? p->in_size0 : 0,
-                            ((p->in_size1 - 1) * p->in_stride1 + 1) * e, p->in_stride0 * e};
-  const RowRegion out_region{p->out_size0, p->out_size1 * p->out_size2 * p->out_size3 * e,
-                             p->out_stride0 * e};
+  const RowRegion in_region =
+      make_region(c, have_input ? p->in_size0 : 0, c.mul(c.add(c.mul(p->in_size1 - 1, p->in_stride1), 1), e),
+                  c.mul(p->in_stride0, e));
+  const RowRegion out_region = make_region(
+      c, p->out_size0, c.mul(c.mul(p->out_size1, p->out_stride1), e), c.mul(p->out_stride0, e));
+  const int64_t in_offset_bytes = c.mul(p->in_offset, e), out_offset_bytes = c.mul(p->out_offset, e);
+  UK_REQUIRE(c.ok && "operand extents fit int64");
   UK_REQUIRE(p->out_size0 == 1 || out_region.pitch >= out_region.width);
 
-  const void* in = (const uint8_t*)p->in_buffer + p->in_offset * e;
-  const void* out = (uint8_t*)p->out_buffer + p->out_offset * e;
+  const void* in = offset_pointer(p->in_buffer, in_offset_bytes);
+  const void* out = offset_pointer(p->out_buffer, out_offset_bytes);
 
   hipStream_t stream = tl_stream;
   Staged s_in, s_out;
@@ -346,9 +439,10 @@ UK_API void iree_uk_pack_p(const iree_uk_pack_params_t* p) {
   // A host input whose rows overlap or interleave (stride0 < row width) is
   // staged as one span.
   RowRegion in_copy = in_region;
-  if (in_copy.rows > 1 && in_copy.pitch < in_copy.width) in_copy = RowRegion{1, in_region.span(), 0};
-  if (!stage_operand(0, in, in_copy, true, stream, &s_in, &d_in)) return;
-  if (!stage_operand(2, out, out_region, false, stream, &s_out, &d_out)) return;
+  if (in_copy.rows > 1 && in_copy.pitch < in_copy.width) in_copy = as_one_span(in_region);
+  Stager stager;
+  if (!stage_operand(stager, 0, in, in_copy, true, stream, &s_in, &d_in)) return;
+  if (!stage_operand(stager, 2, out, out_region, false, stream, &s_out, &d_out)) return;
 
   uk::PackArgs a;
   a.in = (const uint8_t*)d_in;
@@ -404,36 +498,41 @@ UK_API void iree_uk_unpack_p(const iree_uk_unpack_params_t* p) {
   UK_REQUIRE(p->in_size2 >= 0);
   UK_REQUIRE(p->in_size3 >= 0);
   UK_REQUIRE(p->in_stride0 >= 0);
-  UK_REQUIRE(p->in_stride1 == p->in_size2 * p->in_size3);
+  Checked c;
+  UK_REQUIRE(p->in_stride1 == c.mul(p->in_size2, p->in_size3) && c.ok);
   UK_REQUIRE(p->out_stride0 >= 0);
   UK_REQUIRE(p->out_stride1 >= 0);
   int64_t outer0 = p->in_size0, outer1 = p->in_size1;
   int64_t tile0 = p->in_size2, tile1 = p->in_size3;
   if (p->flags & IREE_UK_FLAG_UNPACK_TRANSPOSE_OUTER) { int64_t t = outer0; outer0 = outer1; outer1 = t; }
   if (p->flags & IREE_UK_FLAG_UNPACK_TRANSPOSE_INNER) { int64_t t = tile0; tile0 = tile1; tile1 = t; }
-  UK_REQUIRE(outer0 * tile0 >= p->out_size0);
-  UK_REQUIRE(outer1 * tile1 >= p->out_size1);
+  UK_REQUIRE(tiles_cover(outer0, tile0, p->out_size0));
+  UK_REQUIRE(tiles_cover(outer1, tile1, p->out_size1));
 
   // Early exit of unpack.c:84-86.
   if (p->out_size0 == 0 || p->out_size1 == 0) return;
 
-  const RowRegion in_region{p->in_size0, p->in_size1 * p->in_size2 * p->in_size3 * e,
-                            p->in_stride0 * e};
-  const RowRegion out_region{p->out_size0, ((p->out_size1 - 1) * p->out_stride1 + 1) * e,
-                             p->out_stride0 * e};
+  const RowRegion in_region =
+      make_region(c, p->in_size0, c.mul(c.mul(p->in_size1, p->in_stride1), e), c.mul(p->in_stride0, e));
+  const RowRegion out_region =
+      make_region(c, p->out_size0, c.mul(c.add(c.mul(p->out_size1 - 1, p->out_stride1), 1), e),
+                  c.mul(p->out_stride0, e));
+  const int64_t in_offset_bytes = c.mul(p->in_offset, e), out_offset_bytes = c.mul(p->out_offset, e);
+  UK_REQUIRE(c.ok && "operand extents fit int64");
   UK_REQUIRE(p->in_size0 == 1 || in_region.pitch >= in_region.width);
   UK_REQUIRE(p->out_size0 == 1 || out_region.pitch >= out_region.width);
 
-  const void* in = (const uint8_t*)p->in_buffer + p->in_offset * e;
-  const void* out = (uint8_t*)p->out_buffer + p->out_offset * e;
+  const void* in = offset_pointer(p->in_buffer, in_offset_bytes);
+  const void* out = offset_pointer(p->out_buffer, out_offset_bytes);
 
   hipStream_t stream = tl_stream;
   Staged s_in, s_out;
   const void *d_in, *d_out;
-  if (!stage_operand(0, in, in_region, true, stream, &s_in, &d_in)) return;
+  Stager stager;
+  if (!stage_operand(stager, 0, in, in_region, true, stream, &s_in, &d_in)) return;
   // With an inner output stride the bytes between elements must survive the
   // round trip through the staging buffer, so the rows are uploaded first.
-  if (!stage_operand(2, out, out_region, p->out_stride1 != 1, stream, &s_out, &d_out)) return;
+  if (!stage_operand(stager, 2, out, out_region, p->out_stride1 != 1, stream, &s_out, &d_out)) return;
 
   uk::UnpackArgs a;
   a.in = (const uint8_t*)d_in;

@@ -51,9 +51,6 @@ def load():
     l.iree_uk_mi355x_version.restype = C.c_int
     l.iree_uk_mi355x_multi_mma_i32_16x16x64_i8.argtypes = [vp, vp, vp, C.c_longlong, C.c_longlong] + [C.c_int32] * 6
     l.iree_uk_mi355x_multi_mma_i32_16x16x64_i8.restype = C.c_int
-    l.iree_uk_mi355x_probe_matrix_pipe.argtypes = [C.c_uint32, vp, C.c_longlong, C.c_int, C.c_int,
-                                                   C.POINTER(C.c_double), C.POINTER(C.c_double)]
-    l.iree_uk_mi355x_probe_matrix_pipe.restype = C.c_int
     l.iree_uk_mi355x_init.argtypes = [C.c_int]
     l.iree_uk_mi355x_init.restype = C.c_int
     l.iree_uk_mi355x_set_stream.argtypes = [vp, C.c_int]
@@ -63,3 +60,23 @@ def load():
     l.iree_uk_mi355x_last_kernel.restype = C.c_char_p
     _lib = l
     return l
+
+
+_bench_probe = None
+
+
+def load_bench_probe():
+    """The benchmark's matrix-pipe probe (csrc/bench/probe_matrix_pipe.hip), a
+    helper library of its own: what the matrix pipe sustains on given operand
+    bytes. Not part of the microkernel ABI."""
+    global _bench_probe
+    if _bench_probe is None:
+        path = os.path.join(HERE, "libuk_bench_probe.so")
+        if not os.path.exists(path):
+            raise RuntimeError("%s not found: build it with `python -m iree_amd.build`" % path)
+        l = C.CDLL(path)
+        l.uk_bench_probe_matrix_pipe.argtypes = [C.c_uint32, C.c_void_p, C.c_longlong, C.c_int, C.c_int,
+                                                 C.POINTER(C.c_double), C.POINTER(C.c_double)]
+        l.uk_bench_probe_matrix_pipe.restype = C.c_int
+        _bench_probe = l
+    return _bench_probe

@@ -103,6 +103,26 @@ def test_mmt4d_rejects_what_reference_asserts(kw):
     assert len(f.seen) == 1, kw
 
 
+def test_mmt4d_operand_rows_may_overlap_output_rows_may_not():
+    # The reference puts no condition on strides (mmt4d.c:12-48): a zero or short
+    # lhs/rhs stride is a broadcast or an overlap of rows that are only read.
+    # Rows of the output are written concurrently here, so those must not
+    # overlap; strides that walk backwards are not supported.
+    lib = library.load()
+    buf = (C.c_int8 * 4096)()
+    base = dict(M=2, N=2, K=1, lhs_buffer=C.addressof(buf), rhs_buffer=C.addressof(buf),
+                out_buffer=C.addressof(buf), lhs_stride0=32, rhs_stride0=32, out_stride0=128)
+    for kw in (dict(lhs_stride0=0), dict(rhs_stride0=0), dict(lhs_stride0=8, rhs_stride0=4)):
+        with Failures() as f:
+            lib.iree_uk_mmt4d_p(C.byref(_mmt4d_params(**dict(base, **kw))))
+        # Without a GPU the call fails later, in the HIP runtime; with one it runs.
+        assert not any("stride" in m or "pitch" in m for m in f.seen), f.seen
+    for kw in (dict(out_stride0=64), dict(out_stride0=0), dict(lhs_stride0=-32), dict(rhs_stride0=-32)):
+        with Failures() as f:
+            lib.iree_uk_mmt4d_p(C.byref(_mmt4d_params(**dict(base, **kw))))
+        assert len(f.seen) == 1 and ("stride" in f.seen[0] or "pitch" in f.seen[0]), (kw, f.seen)
+
+
 def test_mmt4d_early_exits_touch_nothing():
     # M == 0, N == 0 and (K == 0 with ACCUMULATE) return before any pointer is
     # looked at (mmt4d.c:105-113): null buffers must be fine, even without a GPU.

@@ -1,0 +1,80 @@
+"""The in-dispatch microkernel in the form the reference's ROCm backend consumes
+its own (compiler/plugins/target/ROCM/builtins/ukernel/CMakeLists.txt:209-218,
+build_tools/cmake/iree_bitcode_library.cmake:273-294): freestanding C23, no
+header outside its directory, compiled to AMDGPU bitcode that defines the
+microkernel (always inlined) and its shared-memory query."""
+import os
+import re
+import subprocess
+
+from iree_amd import build as hip_build
+
+LLVM_DIS = "/opt/rocm/lib/llvm/bin/llvm-dis"
+NAME = hip_build.DEVICE_UKERNEL
+
+
+def test_device_ukernel_source_is_freestanding_c():
+    for fname in os.listdir(hip_build.DEVICE_DIR):
+        text = open(os.path.join(hip_build.DEVICE_DIR, fname)).read()
+        # Only quoted includes of files in the same directory; no C++.
+        for inc in re.findall(r"^\s*#\s*include\s*(.*)$", text, flags=re.M):
+            assert inc.startswith('"') and "/" not in inc, (fname, inc)
+            assert os.path.exists(os.path.join(hip_build.DEVICE_DIR, inc.strip('"'))), (fname, inc)
+        for cxx in ("template", "namespace", "constexpr ", "__host__", "__device__", "hip_runtime"):
+            assert cxx not in text, (fname, cxx)
+
+
+def test_bitcode_builds_and_defines_the_ukernel_and_its_query(tmp_path):
+    out = str(tmp_path / (NAME + ".gfx950.bc"))
+    cmd = [hip_build.CLANG] + hip_build.BITCODE_FLAGS + [os.path.join(hip_build.DEVICE_DIR, NAME + ".c"), "-o", out]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert r.returncode == 0, r.stdout
+    with open(out, "rb") as f:
+        assert f.read(4) == b"BC\xc0\xde"
+    ir = subprocess.run([LLVM_DIS, out, "-o", "-"], stdout=subprocess.PIPE, text=True, check=True).stdout
+    assert 'target triple = "amdgcn-amd-amdhsa"' in ir
+    defs = {name: ret for ret, name in re.findall(r"^define ([^@]*)@([\w.]+)\(", ir, flags=re.M)}
+    assert set(defs) == {NAME, NAME + "_query_shared_memory_bytes"}, defs
+    assert "i32" in defs[NAME + "_query_shared_memory_bytes"] and "void" in defs[NAME]
+    # The same parameter list as the gfx942 microkernel of the reference: 15
+    # parameters, pointers and 64-bit offsets for A, B, C and shared memory.
+    sig = re.search(r"^define [^@]*@%s\((.*)$" % NAME, ir, flags=re.M).group(1)
+    kinds = re.findall(r"\b(ptr|i64|i32) noundef", sig)
+    assert kinds == ["ptr", "i64", "ptr", "i64", "ptr", "i64", "ptr", "i64"] + ["i32"] * 7
+    # always_inline, and the MFMA its name promises.
+    assert re.search(r"attributes #\d+ = \{[^}]*alwaysinline", ir)
+    assert "@llvm.amdgcn.mfma.i32.16x16x64.i8" in ir
+    assert "target-cpu\"=\"gfx950\"" in ir
+    # The query function needs nothing but integer arithmetic: a compiler interprets it at compile time.
+    body = ir[ir.index("@%s_query_shared_memory_bytes(" % NAME):]
+    body = body[:body.index("\n}\n")]
+    assert all("@llvm.smin" in l or "@llvm.smax" in l or "@llvm.umin" in l or "@llvm.umax" in l
+               for l in body.splitlines() if " call " in l), body
+    assert "load " not in body and "store " not in body
+
+
+def test_query_header_matches_known_budgets():
+    # Compile the shared header for the host and evaluate it on the combinations
+    # the wrapper instantiates; the expected numbers follow from the layout:
+    # 16 bytes x staged vectors per step x ring buffers.
+    src = r'''
+#include <stdio.h>
+#include "%s/%s_shared_memory.h"
+int main(void) {
+  static const int c[][5] = {{8,2,8,2,1},{8,2,8,2,2},{4,2,4,2,1},{4,4,4,1,1},{2,1,2,2,1},{2,1,2,1,2},{1,1,2,4,1}};
+  for (unsigned i = 0; i < sizeof c / sizeof c[0]; ++i)
+    printf("%%d\n", get_shared_memory_bytes(get_ab_tile_info(c[i][0] * c[i][4], c[i][1], c[i][3]),
+                                           get_ab_tile_info(c[i][2] * c[i][4], c[i][3], c[i][1])));
+  return 0;
+}''' % (hip_build.DEVICE_DIR, NAME)
+    import tempfile
+    with tempfile.TemporaryDirectory() as d:
+        with open(os.path.join(d, "q.c"), "w") as f:
+            f.write(src)
+        subprocess.run(["gcc", "-std=c11", os.path.join(d, "q.c"), "-o", os.path.join(d, "q")], check=True)
+        got = [int(x) for x in subprocess.run([os.path.join(d, "q")], stdout=subprocess.PIPE, text=True,
+                                              check=True).stdout.split()]
+    # 256x256 tile, K 64: (1024 + 1024) vectors x 16 B = 32 KiB per step, 4 buffers; K 128: 64 KiB, 2 buffers;
+    # 128x128: 16 KiB per step, ring kept within 32 KiB: 2 buffers; only B staged (256 vectors = 4 KiB): 4 buffers;
+    # only A staged (2*64 vectors = 2 KiB): 4 buffers; one subgroup: nothing; narrow A (64 vectors = 1 KiB): 4.
+    assert got == [131072, 131072, 32768, 16384, 8192, 0, 4096]

@@ -1,9 +1,13 @@
 """The in-dispatch int8 microkernel for gfx950
-(iree_amd/csrc/device/iree_uk_amdgpu_multi_mma_mfma_i32_16x16x64_i8.h) through
-its host-callable wrapper: bit-exact against an integer matrix product of the
+(iree_amd/csrc/device/iree_uk_amdgpu_multi_mma_mfma_i32_16x16x64_i8.c, built as
+AMDGPU bitcode and linked into its host-callable wrapper's kernels) through
+that wrapper: bit-exact against an integer matrix product of the
 same operands, for every instantiated parameter combination (tiles staged in
 workgroup memory or read straight from global memory, one or two MFMA K-steps
-per outer step), with accumulation into existing values.
+per outer step, staged tiles smaller than or not a multiple of the workgroup's
+threads, as the reference's heuristics pick them for narrow M:
+GPUEncodingExternalModels.cpp, subgroups 1 x 4), with accumulation into
+existing values.
 
 The data-tiled layouts are those of the reference's gfx942 counterpart
 (compiler/plugins/target/ROCM/builtins/ukernel/
@@ -45,12 +49,13 @@ def untile_c(flat, om, on, SM, SN, IM, IN):
 
 
 @pytest.mark.parametrize("IM,SM,IN,SN,IK", [(8, 2, 8, 2, 1), (8, 2, 8, 2, 2), (4, 2, 4, 2, 1), (4, 4, 4, 1, 1),
-                                             (2, 1, 2, 2, 1), (2, 1, 2, 1, 2)])
+                                             (2, 1, 2, 2, 1), (2, 1, 2, 1, 2), (8, 1, 2, 4, 1), (1, 1, 2, 4, 1),
+                                             (2, 1, 2, 4, 1), (3, 1, 2, 4, 2), (3, 2, 5, 2, 1)])
 @pytest.mark.parametrize("k_size", [1, 2, 5])
 def test_multi_mma_bit_exact(lib, IM, SM, IN, SN, IK, k_size):
     om, on = 3, 2
     rows, cols, depth = om * 16 * IM * SM, on * 16 * IN * SN, k_size * 64 * IK
-    rng = np.random.default_rng(IM * 1000 + SM * 100 + IK * 10 + k_size)
+    rng = np.random.default_rng(IM * 1000 + SM * 100 + IK * 10 + k_size + 7 * SN)
     a = rng.integers(-128, 128, size=(rows, depth), dtype=np.int8)
     b = rng.integers(-128, 128, size=(cols, depth), dtype=np.int8)
     c0 = rng.integers(-1000, 1000, size=(rows, cols), dtype=np.int32)
@@ -69,7 +74,7 @@ def test_multi_mma_bit_exact(lib, IM, SM, IN, SN, IK, k_size):
 def test_multi_mma_rejects_what_is_not_instantiated_and_host_pointers(lib):
     d = torch.zeros(1 << 20, dtype=torch.int8, device="cuda")
     assert lib.iree_uk_mi355x_multi_mma_i32_16x16x64_i8(d.data_ptr(), d.data_ptr(), d.data_ptr(), 1, 1, 1,
-                                                        3, 2, 8, 2, 1) != 0
+                                                        5, 2, 8, 2, 1) != 0
     h = np.zeros(1 << 20, dtype=np.int8)
     assert lib.iree_uk_mi355x_multi_mma_i32_16x16x64_i8(h.ctypes.data, d.data_ptr(), d.data_ptr(), 1, 1, 1,
                                                         8, 2, 8, 2, 1) != 0

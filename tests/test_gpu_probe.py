@@ -1,5 +1,5 @@
-"""The matrix-pipe probe (include/iree_uk_mi355x.h, no counterpart in the
-reference): argument checks, and that its figures are those of an MFMA loop on
+"""The benchmark's matrix-pipe probe (its own helper library, no counterpart in
+the reference): argument checks, and that its figures are those of an MFMA loop on
 this device (below the published int8 peak, at a plausible shader clock, the
 cycle count per step that 32 MFMAs of 8 passes x 4 cycles take)."""
 import ctypes as C
@@ -14,7 +14,7 @@ pytestmark = pytest.mark.gpu
 
 def _probe(lib, buf, traffic, steps=1024, type_flag=abi.MMT4D_TYPE_S8S8S32):
     tops, mhz = C.c_double(), C.c_double()
-    rc = lib.iree_uk_mi355x_probe_matrix_pipe(type_flag, buf.data_ptr(), buf.numel(), traffic, steps,
+    rc = library.load_bench_probe().uk_bench_probe_matrix_pipe(type_flag, buf.data_ptr(), buf.numel(), traffic, steps,
                                               C.byref(tops), C.byref(mhz))
     return rc, tops.value, mhz.value
 
@@ -52,10 +52,10 @@ def test_probe_rejects_bad_arguments():
     buf = torch.zeros(2 << 20, dtype=torch.int8, device="cuda")
     invalid = 1  # hipErrorInvalidValue
     s8 = abi.MMT4D_TYPE_S8S8S32
-    assert lib.iree_uk_mi355x_probe_matrix_pipe(s8, None, 2 << 20, 0, 64, None, None) == invalid
-    assert lib.iree_uk_mi355x_probe_matrix_pipe(s8, buf.data_ptr(), 1 << 20, 0, 64, None, None) == invalid
-    assert lib.iree_uk_mi355x_probe_matrix_pipe(s8, buf.data_ptr(), 2 << 20, 0, 63, None, None) == invalid
-    assert lib.iree_uk_mi355x_probe_matrix_pipe(s8, buf.data_ptr(), 2 << 20, 0, 0, None, None) == invalid
-    assert lib.iree_uk_mi355x_probe_matrix_pipe(abi.MMT4D_TYPE_S8S4S32, buf.data_ptr(), 2 << 20, 0, 64, None, None) == invalid
+    assert library.load_bench_probe().uk_bench_probe_matrix_pipe(s8, None, 2 << 20, 0, 64, None, None) == invalid
+    assert library.load_bench_probe().uk_bench_probe_matrix_pipe(s8, buf.data_ptr(), 1 << 20, 0, 64, None, None) == invalid
+    assert library.load_bench_probe().uk_bench_probe_matrix_pipe(s8, buf.data_ptr(), 2 << 20, 0, 63, None, None) == invalid
+    assert library.load_bench_probe().uk_bench_probe_matrix_pipe(s8, buf.data_ptr(), 2 << 20, 0, 0, None, None) == invalid
+    assert library.load_bench_probe().uk_bench_probe_matrix_pipe(abi.MMT4D_TYPE_S8S4S32, buf.data_ptr(), 2 << 20, 0, 64, None, None) == invalid
     # Output pointers are optional.
-    assert lib.iree_uk_mi355x_probe_matrix_pipe(s8, buf.data_ptr(), 2 << 20, 1, 64, None, None) == 0
+    assert library.load_bench_probe().uk_bench_probe_matrix_pipe(s8, buf.data_ptr(), 2 << 20, 1, 64, None, None) == 0
