@@ -249,6 +249,26 @@ int iree_uk_mi355x_multi_mma_i32_16x16x64_i8(const void* a, const void* b, void*
                                              int32_t subgroups_m, int32_t intrinsics_n, int32_t subgroups_n,
                                              int32_t intrinsics_k);
 
+/* iree_uk_mmt4d_p for callers that cannot allocate. It has no counterpart in
+ * the reference (whose microkernels never allocate, being CPU code); it is for
+ * callers that may not call hipMalloc where they call a microkernel: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid
+ * allocation. Same parameters, checks, kernels and results as iree_uk_mmt4d_p.
+ * The difference: operands at host addresses are mirrored in a fixed array of
+ * IREE_UK_MI355X_NOALLOC_MAX_STAGED_BYTES of device memory that the library's
+ * code object holds on every device it runs on until the process ends, instead
+ * of in staging buffers grown with hipMalloc. Each host operand takes its span
+ * (first to last touched byte) rounded up to 256 bytes; a call whose host
+ * operands need more in total reports "host operands exceed ..." through the
+ * failure handler and returns without launching. Device operands take none.
+ * The call makes no hipMalloc/hipFree. All calls on one device share that
+ * array: calls that overlap in time on one device race (serialise them); the
+ * array keeps the previous call's bytes, and nothing read from it is ever
+ * older than the current call's own uploads. iree_uk_mi355x_init resolves
+ * the array's address ahead of the first call. */
+#define IREE_UK_MI355X_NOALLOC_MAX_STAGED_BYTES (16 * 1024 * 1024)
+void iree_uk_mi355x_mmt4d_noalloc_p(const iree_uk_mmt4d_params_t* params);
+
 /* Library version, MAJOR*10000 + MINOR*100 + PATCH. */
 int iree_uk_mi355x_version(void);
 

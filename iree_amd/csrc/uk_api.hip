@@ -100,12 +100,62 @@ struct StageBuffer {
 };
 thread_local StageBuffer tl_stage[3];
 
-// Where the calling entry point mirrors host operands.
+// Static staging memory of the allocation-free entry point: one array per
+// device, owned by the code object, resolved to a device address once per
+// device (the array's name is only a host-side handle for that lookup).
+constexpr size_t kScratchBytes = (size_t)IREE_UK_MI355X_NOALLOC_MAX_STAGED_BYTES;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+std::atomic<unsigned char*> g_scratch_ptr[kMaxDevices];
+
+// Device address of the current device's `scratch` (nullptr after reporting
+// a failure).
+unsigned char* scratch_for_current_device() {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  unsigned char* ptr = g_scratch_ptr[device].load(std::memory_order_acquire);
+  if (ptr) return ptr;
+  void* resolved = nullptr;
+  if (hipGetSymbolAddress(&resolved, HIP_SYMBOL(scratch)) != hipSuccess || !resolved) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  // Two threads racing here resolve the same address.
+  g_scratch_ptr[device].store((unsigned char*)resolved, std::memory_order_release);
+  return (unsigned char*)resolved;
+}
+
+// Where the calling entry point mirrors host operands: the thread's grow-only
+// buffers (may call hipMalloc), or a bump allocator over the device's static
+// scratch (never allocates; fails when the operands do not fit).
 struct Stager {
+  unsigned char* fixed_base = nullptr;  // non-null: static scratch
+  size_t fixed_used = 0;
+  bool no_alloc = false;
 };
 
 bool stage_reserve(Stager& stager, int slot, size_t bytes, void** out) {
-  (void)stager;
+  if (stager.no_alloc) {
+    if (!stager.fixed_base) {
+      stager.fixed_base = scratch_for_current_device();
+      if (!stager.fixed_base) {
+        report_failure(__FILE__, __LINE__, __func__, "hipGetSymbolAddress(scratch) failed on the current device");
+        return false;
+      }
+    }
+    const size_t rounded = (bytes + 255) & ~(size_t)255;
+    if (rounded > kScratchBytes - stager.fixed_used) {
+      report_failure(__FILE__, __LINE__, __func__,
+                     "host operands exceed IREE_UK_MI355X_NOALLOC_MAX_STAGED_BYTES of static staging memory");
+      return false;
+    }
+    *out = stager.fixed_base + stager.fixed_used;
+    stager.fixed_used += rounded;
+    return true;
+  }
   StageBuffer& s = tl_stage[slot];
   if (s.capacity < bytes) {
     if (s.ptr) UK_HIP_OK(hipFree(s.ptr));
@@ -346,6 +396,12 @@ void mmt4d_impl(const iree_uk_mmt4d_params_t* p, Stager& stager) {
 
 UK_API void iree_uk_mmt4d_p(const iree_uk_mmt4d_params_t* p) {
   Stager stager;
+  mmt4d_impl(p, stager);
+}
+
+UK_API void iree_uk_mi355x_mmt4d_noalloc_p(const iree_uk_mmt4d_params_t* p) {
+  Stager stager;
+  stager.no_alloc = true;
   mmt4d_impl(p, stager);
 }
 
@@ -625,6 +681,11 @@ UK_API int iree_uk_mi355x_init(int device_ordinal) {
   e = hipGetDeviceProperties(&prop, device_ordinal);
   if (e != hipSuccess) return (int)e;
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return (int)hipErrorInvalidDevice;
+  // Resolve this device's static staging memory now, so that the
+  // allocation-free entry point does nothing but copies and launches.
+  if (device_ordinal < kMaxDevices && hipSetDevice(device_ordinal) == hipSuccess &&
+      !scratch_for_current_device())
+    return (int)hipErrorInvalidSymbol;
   return 0;
 }
 

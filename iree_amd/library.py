@@ -31,6 +31,8 @@ def load():
     l.iree_uk_mmt4d.restype = None
     l.iree_uk_mmt4d_p.argtypes = [C.POINTER(abi.Mmt4dParams)]
     l.iree_uk_mmt4d_p.restype = None
+    l.iree_uk_mi355x_mmt4d_noalloc_p.argtypes = [C.POINTER(abi.Mmt4dParams)]
+    l.iree_uk_mi355x_mmt4d_noalloc_p.restype = None
     l.iree_uk_mmt4d_info.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_uint32, u64p]
     l.iree_uk_mmt4d_info.restype = C.c_uint32
     l.iree_uk_mmt4d_info_p.argtypes = [C.POINTER(abi.Mmt4dParams)]
