@@ -107,9 +107,73 @@ def _headline(torch, lib, abi, synth, steps, warmup):
                          "accumulate off, operands resident in HBM")
 
 
+def _e2e_chain(torch, lib, abi, synth, steps, warmup):
+    """The chain the reference's matmul benchmark runs (tools/e2e_matmul_benchmark.c:173-186):
+    pack lhs, pack rhs (given as [K, N], both transposes), mmt4d, unpack, on row-major int8
+    4096x4096 operands, with the tile sizes iree_uk_query_tile_sizes_2d hands out. One step =
+    the four calls; checked against the sum of the row-major product (column sums of A times
+    row sums of B)."""
+    def tiles(role):
+        q, o = abi.QueryTileSizes2dParams(), abi.QueryTileSizes2dOutParams()
+        q.flags = abi.QTS_OP_MATMUL_I8I8I32 | role
+        lib.iree_uk_query_tile_sizes_2d(C.byref(q), C.byref(o))
+        return o.tile_size0, o.tile_size1
+    (m0, k0), (n0, _) = tiles(abi.QTS_ROLE_LHS), tiles(abi.QTS_ROLE_RHS)
+    S = 4096
+    a = torch.from_numpy(synth.uniform_int8(21, 0, S * S)).cuda()      # A [M, K]
+    b = torch.from_numpy(synth.uniform_int8(21, 1, S * S)).cuda()      # B [K, N]
+    M1, N1, K1 = S // m0, S // n0, S // k0
+    a4, b4 = torch.empty_like(a), torch.empty_like(b)
+    c4 = torch.empty(S * S, dtype=torch.int32, device="cuda")
+    c = torch.empty(S * S, dtype=torch.int32, device="cuda")
+
+    def pack(src, dst, rows, cols, o0, o1, t0, t1, flags):
+        p = abi.PackParams()
+        p.in_buffer, p.out_buffer = src.data_ptr(), dst.data_ptr()
+        p.in_stride0, p.in_stride1, p.in_size0, p.in_size1 = cols, 1, rows, cols
+        p.out_size0, p.out_size1, p.out_size2, p.out_size3 = o0, o1, t0, t1
+        p.out_stride0, p.out_stride1 = o1 * t0 * t1, t0 * t1
+        p.flags = abi.PACK_TYPE_I8I8 | flags
+        return p
+    p_lhs = pack(a, a4, S, S, M1, K1, m0, k0, 0)
+    p_rhs = pack(b, b4, S, S, N1, K1, n0, k0, abi.PACK_TRANSPOSE_INNER | abi.PACK_TRANSPOSE_OUTER)
+    p_mm = _mmt4d_params(abi, a4.data_ptr(), b4.data_ptr(), c4.data_ptr(), M1, N1, K1, m0, n0, k0,
+                         abi.MMT4D_TYPE_S8S8S32)
+    u = abi.UnpackParams()
+    u.in_buffer, u.out_buffer = c4.data_ptr(), c.data_ptr()
+    u.in_size0, u.in_size1, u.in_size2, u.in_size3 = M1, N1, m0, n0
+    u.in_stride0, u.in_stride1 = N1 * m0 * n0, m0 * n0
+    u.out_size0, u.out_size1, u.out_stride0, u.out_stride1 = S, S, S, 1
+    u.flags = abi.UNPACK_TYPE_I32I32
+    parts = {}
+
+    def timed(name, fn):
+        ms, _ = _time_launches(torch, fn, steps, warmup)
+        parts[name] = {"ms": round(ms, 5), "kernel": lib.iree_uk_mi355x_last_kernel().decode()}
+    timed("pack_lhs", lambda: lib.iree_uk_pack_p(C.byref(p_lhs)))
+    timed("pack_rhs_transposed", lambda: lib.iree_uk_pack_p(C.byref(p_rhs)))
+    timed("mmt4d", lambda: lib.iree_uk_mmt4d_p(C.byref(p_mm)))
+    timed("unpack", lambda: lib.iree_uk_unpack_p(C.byref(u)))
+
+    def chain():
+        lib.iree_uk_pack_p(C.byref(p_lhs))
+        lib.iree_uk_pack_p(C.byref(p_rhs))
+        lib.iree_uk_mmt4d_p(C.byref(p_mm))
+        lib.iree_uk_unpack_p(C.byref(u))
+    ms, _ = _time_launches(torch, chain, steps, warmup)
+    want = (a.view(S, S).to(torch.int64).sum(dim=0) * b.view(S, S).to(torch.int64).sum(dim=1)).sum().item()
+    rows = [0, 1777, 4095]
+    ref_rows = (a.view(S, S)[rows].double() @ b.view(S, S).double()).long()
+    ok = bool(c.to(torch.int64).sum().item() == want) and bool(torch.equal(c.view(S, S)[rows].long(), ref_rows))
+    return {"tiles": "%dx%dx%d" % (m0, n0, k0), "ms": round(ms, 5), "value": round(2.0 * S ** 3 / ms / 1e9, 1),
+            "unit": "TOP/s", "frac_of_peak": round(2.0 * S ** 3 / ms / 1e9 / PEAK_INT8_TOPS, 4),
+            "equals_row_major_product": ok, "parts": parts}
+
+
 def _also(torch, lib, abi, synth, steps, warmup):
     """One-launch figures for the other configurations."""
     import numpy as np
+    from iree_amd import library
     res = {}
 
     def mm(name, flags, M, N, K, M0, N0, K0, lhs, rhs, out_dtype, peak, unit, acc=False, bytes_model=None):
@@ -157,6 +221,24 @@ def _also(torch, lib, abi, synth, steps, warmup):
     mm("mmt4d_s8s8s32_4096_8x8x4_all_zero_operands_clock_check", abi.MMT4D_TYPE_S8S8S32, 512, 512, 1024, 8, 8, 4,
        zl, zl, torch.int32, PEAK_INT8_TOPS, "TOP/s")
     del zl
+    # A second opinion on what this part does on this problem: the vendor's own
+    # int8 GEMM (torch._int_mm -> hipBLASLt) on the same logical 4096^3 with
+    # uniformly random int8, row-major operands. Not a result of this library.
+    try:
+        va = torch.from_numpy(synth.uniform_int8(0, 0, n)).cuda().view(4096, 4096)
+        vb = torch.from_numpy(synth.uniform_int8(0, 1, n)).cuda().view(4096, 4096)
+        best = None
+        for operand in (vb, vb.t()):
+            ms, _ = _time_launches(torch, lambda: torch._int_mm(va, operand), steps, warmup)
+            best = ms if best is None else min(best, ms)
+        res["vendor_library_int8_gemm_4096_for_comparison"] = {
+            "what": "torch._int_mm (hipBLASLt), best of B and B^T layouts", "ms": round(best, 5),
+            "value": round(2.0 * 4096 ** 3 / best / 1e9, 1), "unit": "TOP/s",
+            "frac_of_peak": round(2.0 * 4096 ** 3 / best / 1e9 / PEAK_INT8_TOPS, 4)}
+        del va, vb
+    except Exception as exc:  # not every torch build has it
+        res["vendor_library_int8_gemm_4096_for_comparison"] = {"unavailable": str(exc)[:200]}
+    res["e2e_pack_mmt4d_unpack_s8s8s32_4096"] = _e2e_chain(torch, lib, abi, synth, steps, warmup)
     # What the matrix pipe sustains on this device, measured by the
     # benchmark's probe (a helper library of its own): the 256x256 kernel's inner-loop instruction mix with no
     # HBM traffic, no prologue and no epilogue, on all-zero bytes, on the
@@ -483,6 +565,79 @@ def _cpu_baseline(abi, synth, threads):
     return base, extra
 
 
+def _cpu_baseline_other_configs(abi, synth, threads):
+    """The compiled reference on this host for the other configurations, in the tile shapes of
+    the configurations themselves (no x86-64 tile exists for any of them: generic tile
+    functions, mmt4d_tile_generic.c) and in the reference's own x86-64 tile shapes
+    (arch/x86_64/mmt4d_x86_64_tiles.inl). Each entry says whether the reference selected an
+    architecture-specific tile function on this host. Bounded samples where the generic
+    functions would take minutes."""
+    import numpy as np
+    import oracle
+    ref = oracle.ref_lib()
+    if ref is None:
+        return None
+    cpu = oracle.host_cpu_data()
+    rows = {}
+
+    def run(name, flags, M, N, K, M0, N0, K0, lhs, rhs, out, sample, unit="TFLOP/s", nbytes=None, reps=2):
+        p = _mmt4d_params(abi, lhs.ctypes.data, rhs.ctypes.data, out.ctypes.data, M, N, K, M0, N0, K0,
+                          flags | abi.MMT4D_ALLOW_GENERIC_FALLBACK)
+        p.cpu_data = C.cast(cpu, C.POINTER(C.c_uint64))
+        arch = bool(ref.ref_mmt4d_info(C.byref(p)) & 1)
+        best = None
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            ref.ref_mmt4d_mt(C.byref(p), threads)
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        ops = 2.0 * M * N * K * M0 * N0 * K0
+        entry = {"value": round(ops / best / 1e12, 5), "unit": unit, "cores": threads, "kind": "reference",
+                 "arch_tile_selected": arch, "seconds": round(best, 4), "sample": sample}
+        if nbytes is not None:
+            entry.update({"value": round(nbytes / best / 1e9, 2), "unit": "GB/s", "gflops": round(ops / best / 1e9, 2)})
+        rows[name] = entry
+
+    def f16(seed, stream, n, sigma, bf16=False):
+        x = synth.normal_f32(seed, stream, n, sigma)
+        return synth.bf16_bits(x) if bf16 else synth.f16_bits(x)
+
+    n = 4096 * 4096
+    h_l, h_r = f16(3, 0, n, 1.0 / 64), f16(3, 1, n, 1.0 / 64)
+    acc = synth.normal_f32(3, 2, n)
+    # f16f16f32 4096^3 with accumulate: the reference's x86-64 shape 16x16x1 (whole problem) and the
+    # configuration's own 16x16x16 (generic; 16 of its 256 rows of tiles).
+    run("mmt4d_f16f16f32_4096_x86_tile_16x16x1_acc", abi.MMT4D_TYPE_F16F16F32 | abi.MMT4D_ACCUMULATE, 256, 256, 4096,
+        16, 16, 1, h_l, h_r, acc.copy(), "whole 4096^3, best of 2")
+    run("mmt4d_f16f16f32_4096_16x16x16_acc", abi.MMT4D_TYPE_F16F16F32 | abi.MMT4D_ACCUMULATE, 16, 256, 256, 16, 16, 16,
+        h_l, h_r, acc.copy(), "rows 0..15 of the 256 rows of lhs tiles (1/16 of the workload), best of 1", reps=1)
+    del h_l, h_r, acc
+    b_l, b_r = f16(4, 0, n, 1.0, bf16=True), f16(4, 10, n, 0.02, bf16=True)
+    run("mmt4d_bf16bf16f32_4096_x86_tile_16x16x2", abi.MMT4D_TYPE_BF16BF16F32, 256, 256, 2048, 16, 16, 2, b_l, b_r,
+        np.zeros(n, np.float32), "whole 4096^3, best of 2")
+    del b_l, b_r
+    # bf16 matrix-vector shapes, N = 14336, K = 4096 (rhs panels split over the threads).
+    nk = 14336 * 4096
+    w = f16(4, 10, nk, 0.02, bf16=True)
+    x1 = f16(4, 1, 4096, 1.0, bf16=True)
+    run("mmt4d_bf16_skinny_x86_tile_1x16x2_N14336_K4096", abi.MMT4D_TYPE_BF16BF16F32, 1, 896, 2048, 1, 16, 2, x1, w,
+        np.zeros(14336, np.float32), "whole workload, best of 3", nbytes=nk * 2 + 4096 * 2 + 14336 * 4, reps=3)
+    for m0 in (1, 16):
+        xm = f16(4, m0, m0 * 4096, 1.0, bf16=True)
+        run("mmt4d_bf16_skinny_M%d_N14336_K4096_%dx16x8" % (m0, m0), abi.MMT4D_TYPE_BF16BF16F32, 1, 896 // 4, 512, m0, 16,
+            8, xm, w, np.zeros(14336 * m0 // 4, np.float32),
+            "the first 224 of the 896 rhs panels (1/4 of the workload), best of 1",
+            nbytes=(nk * 2) // 4 + m0 * 4096 * 2 + 14336 * m0, reps=1)
+    del w
+    # s8s4s32 512 x 11008 x 4096, tiles 16x16x32: no architecture-specific tile in the reference.
+    lhs = synth.uniform_int8(5, 0, 512 * 4096)
+    rhs = synth.uniform_int4_packed(5, 1, 11008 * 4096)
+    run("mmt4d_s8s4s32_512x11008x4096_16x16x32", abi.MMT4D_TYPE_S8S4S32, 32, 688 // 4, 128, 16, 16, 32, lhs,
+        rhs.view(np.int8), np.zeros(512 * 11008 // 4, np.int32),
+        "the first 172 of the 688 rhs panels (1/4 of the workload), best of 1", unit="TOP/s", reps=1)
+    return rows
+
+
 def _cpu_pack_unpack(abi, synth, threads):
     """The reference's pack and unpack on this host (f32 [8191, 8190] <-> [512, 8190, 16, 1],
     rows of tiles split over `threads`), GB/s counted like the GPU figures (read + written)."""
@@ -595,8 +750,14 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(tops, 2), "peak": PEAK_INT8_TOPS,
                      "unit": "TOP/s", "frac": round(tops / PEAK_INT8_TOPS, 4),
                      "traffic": HEADLINE_TRAFFIC_BYTES,
-                     "kernel_ms": round(head["ev_ms"], 5),
-                     "kernel_ms_median": round(head["med_ms"], 5), "kernel_ms_min": round(head["min_ms"], 5)},
+                     "traffic_source": "profiles/bench_all_workloads_hbm_traffic.txt (rocprofv3 FETCH_SIZE, "
+                                       "WRITE_SIZE of this command, scaled by a plain copy; not measured in this run)",
+                     # `achieved` = ops / this: the mean over the timed steps, launched back to back,
+                     # between two HIP events on the launch stream.
+                     "kernel_ms_mean_back_to_back": round(head["ev_ms"], 5),
+                     # Each launch between its own pair of events (includes the events' own gaps).
+                     "kernel_ms_single_launch_median": round(head["med_ms"], 5),
+                     "kernel_ms_single_launch_min": round(head["min_ms"], 5)},
         "cpu_baseline": cpu,
     }
     if cpu_arch is not None:
@@ -605,6 +766,9 @@ def main():
         cpu_pack = _cpu_pack_unpack(abi, synth, threads)
         if cpu_pack is not None:
             line["cpu_baseline_pack_unpack"] = cpu_pack
+        cpu_other = _cpu_baseline_other_configs(abi, synth, threads)
+        if cpu_other is not None:
+            line["cpu_baseline_other_configs"] = cpu_other
     if also is not None:
         line["also"] = also
     print(json.dumps(line))

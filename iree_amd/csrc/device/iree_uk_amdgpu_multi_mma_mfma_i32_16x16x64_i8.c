@@ -170,6 +170,9 @@ static inline void issue_tile_loads(uint32_t lds_address, const int32x4_t *tile_
   // Load existing accumulators from global memory into registers. The VLAs
   // become normal arrays after inlining.
   int32x4_t c_regs[intrinsics_m][intrinsics_n];
+  // One K-step's B operands. (Declared here, not inside the loops: a variable
+  // length array in a loop stays a stack allocation after inlining.)
+  int32x4_t b_regs[intrinsics_n];
   for (int m = 0; m < intrinsics_m; ++m) {
     for (int n = 0; n < intrinsics_n; ++n) {
       c_regs[m][n] = c_global[64 * (m * intrinsics_n + n)];
@@ -221,7 +224,6 @@ static inline void issue_tile_loads(uint32_t lds_address, const int32x4_t *tile_
                                   ? shared + buffer * shared_vecs + a_tile.num_shared_vecs + b_thread_relative_offset
                                   : b_global + (int64_t)k_outer * b_tile.num_vecs;
     for (int k = 0; k < intrinsics_k; ++k) {
-      int32x4_t b_regs[intrinsics_n];
       for (int n = 0; n < intrinsics_n; ++n) {
         b_regs[n] = b_vecs[64 * intrinsics_k * n + k];
       }

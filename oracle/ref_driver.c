@@ -8,8 +8,9 @@
  *   - iree_uk_assert_fail (declared extern at common.h:307-309),
  *   - ref_host_cpu_data: the x86-64 feature words the reference's tile
  *     selection reads (bit positions from schemas/cpu_feature_bits.inl:85-117),
- *   - ref_*_mt: static split of the outer M (rows of tiles) dimension over
- *     pthreads, each thread calling the reference entry point on its slice,
+ *   - ref_*_mt: static split of the outer M (rows of tiles) dimension (of N
+ *     for matrix-vector shapes) over pthreads, each thread calling the
+ *     reference entry point on its slice,
  *     which is the decomposition the reference's CPU backend applies when it
  *     distributes a dispatch over workgroups.
  * Parameter structs are declared from this repository's header; the layouts are
@@ -98,17 +99,26 @@ static void run_jobs(job_t* jobs, int n) {
 
 static int clamp_threads(int threads) { return threads < 1 ? 1 : (threads > 256 ? 256 : threads); }
 
-/* mmt4d with rows of tiles [M*t/T, M*(t+1)/T) on thread t. */
+/* mmt4d with rows of tiles [M*t/T, M*(t+1)/T) on thread t; with fewer rows of
+ * tiles than threads (matrix-vector shapes) the rhs panels are split instead. */
 REF_EXPORT void ref_mmt4d_mt(const iree_uk_mmt4d_params_t* p, int threads) {
   threads = clamp_threads(threads);
   job_t* jobs = (job_t*)calloc(threads, sizeof(job_t));
+  const int split_n = p->M < threads && p->N > p->M;
   for (int t = 0; t < threads; ++t) {
-    const int64_t b = p->M * t / threads, e = p->M * (t + 1) / threads;
     jobs[t].kind = 0;
     jobs[t].mm = *p;
-    jobs[t].mm.M = e - b;
-    jobs[t].mm.lhs_offset = p->lhs_offset + b * p->lhs_stride0;
-    jobs[t].mm.out_offset = p->out_offset + b * p->out_stride0;
+    if (split_n) {
+      const int64_t b = p->N * t / threads, e = p->N * (t + 1) / threads;
+      jobs[t].mm.N = e - b;
+      jobs[t].mm.rhs_offset = p->rhs_offset + b * p->rhs_stride0;
+      jobs[t].mm.out_offset = p->out_offset + b * p->M0 * p->N0;
+    } else {
+      const int64_t b = p->M * t / threads, e = p->M * (t + 1) / threads;
+      jobs[t].mm.M = e - b;
+      jobs[t].mm.lhs_offset = p->lhs_offset + b * p->lhs_stride0;
+      jobs[t].mm.out_offset = p->out_offset + b * p->out_stride0;
+    }
   }
   run_jobs(jobs, threads);
   free(jobs);
