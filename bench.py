@@ -508,6 +508,79 @@ def _also(torch, lib, abi, synth, steps, warmup):
     return res
 
 
+def _power_clock_samples(torch, lib, abi, synth, seconds):
+    """Socket power and shader clocks (amd-smi, polled from a thread) while the headline
+    kernel runs back to back for `seconds`: on its uniformly random int8, on all-zero
+    operands (same instruction stream and traffic), and the vendor's int8 GEMM on the same
+    logical problem. Shows what the part sustains on this data; not a result."""
+    import subprocess
+    import threading
+    import numpy as np
+
+    def poll(stop, out):
+        while not stop.is_set():
+            try:
+                r = subprocess.run(["amd-smi", "metric", "-p", "-c", "--json"], stdout=subprocess.PIPE,
+                                   stderr=subprocess.DEVNULL, text=True, timeout=10)
+                d = json.loads(r.stdout)
+                g = d[0] if isinstance(d, list) else d.get("gpu_data", [d])[0]
+                value = lambda x: float(x["value"] if isinstance(x, dict) else x)
+                clocks = [value(v["clk"]) for k, v in g["clock"].items() if k.startswith("gfx_")]
+                out.append((value(g["power"]["socket_power"]), clocks))
+            except Exception:  # tool missing or another output format: no samples
+                time.sleep(0.5)
+
+    def loop(name, fn, ops):
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+        stop, samples = threading.Event(), []
+        th = threading.Thread(target=poll, args=(stop, samples))
+        th.start()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0, launches = time.time(), 0
+        e0.record()
+        while time.time() - t0 < seconds:
+            for _ in range(200):
+                fn()
+            launches += 200
+            torch.cuda.synchronize()
+        e1.record()
+        torch.cuda.synchronize()
+        stop.set()
+        th.join()
+        ms = e0.elapsed_time(e1) / launches
+        samples = samples[1:] if len(samples) > 2 else samples   # the first may predate the loop
+        power = [s[0] for s in samples]
+        clock = [float(np.mean(s[1])) for s in samples if s[1]]
+        return {"loop": name, "launches": launches, "ms_per_launch": round(ms, 5),
+                "value": round(ops / ms / 1e9, 1), "unit": "TOP/s", "frac_of_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS, 4),
+                "samples": len(samples),
+                "socket_power_W_mean": round(float(np.mean(power)), 1) if power else None,
+                "socket_power_W_max": round(float(np.max(power)), 1) if power else None,
+                "shader_clock_MHz_mean_over_xcds": round(float(np.mean(clock))) if clock else None,
+                "shader_clock_MHz_min": round(float(np.min(clock))) if clock else None}
+
+    n = 4096 * 4096
+    ops = 2.0 * 4096 ** 3
+    out = torch.empty(n, dtype=torch.int32, device="cuda")
+
+    def headline_on(l, r):
+        p = _mmt4d_params(abi, l.data_ptr(), r.data_ptr(), out.data_ptr(), 512, 512, 1024, 8, 8, 4, abi.MMT4D_TYPE_S8S8S32)
+        return lambda: lib.iree_uk_mmt4d_p(C.byref(p))
+    rl = torch.from_numpy(synth.uniform_int8(0, 0, n)).cuda()
+    rr = torch.from_numpy(synth.uniform_int8(0, 1, n)).cuda()
+    zeros = torch.zeros(n, dtype=torch.int8, device="cuda")
+    rows = [loop("mmt4d s8s8s32 4096^3 8x8x4, uniform random int8 (the headline)", headline_on(rl, rr), ops),
+            loop("the same launch on all-zero operands", headline_on(zeros, zeros), ops)]
+    try:
+        a2, b2 = rl.view(4096, 4096), rr.view(4096, 4096).t()
+        rows.append(loop("torch._int_mm 4096^3 (hipBLASLt), uniform random int8", lambda: torch._int_mm(a2, b2), ops))
+    except Exception:
+        pass
+    return rows
+
+
 def _cpu_baseline(abi, synth, threads):
     """The reference CPU ukernels (compiled from the reference's own sources into
     oracle/_ref) on this host; falls back to this repository's scalar port."""
@@ -690,6 +763,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-also", action="store_true", help="headline workload only")
+    ap.add_argument("--sample-power", type=float, default=0.0, metavar="SECONDS",
+                    help="also loop the headline kernel for SECONDS per data set while polling amd-smi for "
+                         "socket power and shader clocks (adds `power_clock_samples` to the line)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device-to-device copy three times (a kernel of "
                          "known traffic, to scale the profiler's FETCH_SIZE / WRITE_SIZE readings)")
@@ -771,6 +847,10 @@ def main():
             line["cpu_baseline_other_configs"] = cpu_other
     if also is not None:
         line["also"] = also
+    if args.sample_power > 0:
+        lib.iree_uk_mi355x_set_stream(torch.cuda.current_stream().cuda_stream, 1)
+        line["power_clock_samples"] = _power_clock_samples(torch, lib, abi, synth, args.sample_power)
+        lib.iree_uk_mi355x_set_stream(None, 0)
     print(json.dumps(line))
 
 

@@ -254,59 +254,83 @@ __device__ __forceinline__ void store_block(const MfmaArgs& a, typename AccType<
       return v;
     }
   };
+  // With paired lhs fragments, fragments 2p and 2p + 1 hold the even and the odd
+  // rows of the same 64: they are written together, so that the stores which
+  // make up a cache line of the output (two rows of a 16-wide int32 tile, say)
+  // follow each other directly. Written a fragment at a time, each line was
+  // sent to memory in pieces (2.6x the output size in write traffic).
+  constexpr int IS = PAIR_A ? 2 : 1;  // lhs fragments written together
 #pragma unroll
-  for (int i = 0; i < AM; ++i) {
-    const int64_t this_row =
-        wave_row + (PAIR_A ? 64 * (i >> 1) + 2 * (lane & 31) + (i & 1) : 32 * i + (lane & 31));
-    const int64_t row = min(this_row, total_rows - 1);
-    const bool row_inside = this_row < total_rows;
-    uint8_t* row_out =
-        wave_out + OUT_BYTES * ((row >> a.log2_M0) * a.out_stride0 + ((row & (M0 - 1)) << a.log2_N0));
+  for (int i0 = 0; i0 < AM; i0 += IS) {
+    bool row_inside[IS];
+    uint8_t* row_out[IS];
+#pragma unroll
+    for (int t = 0; t < IS; ++t) {
+      const int i = i0 + t;
+      const int64_t this_row =
+          wave_row + (PAIR_A ? 64 * (i >> 1) + 2 * (lane & 31) + (i & 1) : 32 * i + (lane & 31));
+      const int64_t row = min(this_row, total_rows - 1);
+      row_inside[t] = this_row < total_rows;
+      row_out[t] = wave_out + OUT_BYTES * ((row >> a.log2_M0) * a.out_stride0 + ((row & (M0 - 1)) << a.log2_N0));
+    }
 #pragma unroll
     for (int j0 = 0; j0 < BN; j0 += JS) {
       // Pin the fragment(s) where they are until their turn: left alone, the
       // compiler moves all 256 accumulators to ordinary registers right after
       // the main loop, and there are not that many.
-      typename AccType<KIND>::type frag[JS];
+      typename AccType<KIND>::type frag[IS][JS];
 #pragma unroll
-      for (int s = 0; s < JS; ++s) {
-        frag[s] = acc[i][j0 + s];
-        asm volatile("" : "+a"(frag[s]));
-      }
-      quad_t v[JS][4];
+      for (int t = 0; t < IS; ++t)
 #pragma unroll
-      for (int s = 0; s < JS; ++s)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          if constexpr (PAIR_B) {
-            v[s][q] = quad_t{frag[0][4 * q + 2 * s], frag[1][4 * q + 2 * s], frag[0][4 * q + 2 * s + 1],
-                             frag[1][4 * q + 2 * s + 1]};
-          } else {
-            v[s][q] = quad_t{frag[s][4 * q], frag[s][4 * q + 1], frag[s][4 * q + 2], frag[s][4 * q + 3]};
-          }
-          if constexpr (RHS_I4) v[s][q] = v[s][q] >> 4;
+        for (int s = 0; s < JS; ++s) {
+          frag[t][s] = acc[i0 + t][j0 + s];
+          asm volatile("" : "+a"(frag[t][s]));
         }
-      if (a.accumulate) {
-        quad_t old[JS][4];
+      quad_t v[IS][JS][4];
+#pragma unroll
+      for (int t = 0; t < IS; ++t)
 #pragma unroll
         for (int s = 0; s < JS; ++s)
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            old[s][q] = quad_t{0, 0, 0, 0};
-            if (row_inside && (col_inside >> (4 * (j0 + s) + q) & 1))
-              old[s][q] = to_float(*(const stored_t*)(row_out + col_off[j0 + s][q]));
+            if constexpr (PAIR_B) {
+              v[t][s][q] = quad_t{frag[t][0][4 * q + 2 * s], frag[t][1][4 * q + 2 * s], frag[t][0][4 * q + 2 * s + 1],
+                                  frag[t][1][4 * q + 2 * s + 1]};
+            } else {
+              v[t][s][q] = quad_t{frag[t][s][4 * q], frag[t][s][4 * q + 1], frag[t][s][4 * q + 2], frag[t][s][4 * q + 3]};
+            }
+            if constexpr (RHS_I4) v[t][s][q] = v[t][s][q] >> 4;
           }
+      if (a.accumulate) {
+        quad_t old[IS][JS][4];
 #pragma unroll
-        for (int s = 0; s < JS; ++s)
+        for (int t = 0; t < IS; ++t)
 #pragma unroll
-          for (int q = 0; q < 4; ++q) v[s][q] += old[s][q];
+          for (int s = 0; s < JS; ++s)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              old[t][s][q] = quad_t{0, 0, 0, 0};
+              if (row_inside[t] && (col_inside >> (4 * (j0 + s) + q) & 1))
+                old[t][s][q] = to_float(*(const stored_t*)(row_out[t] + col_off[j0 + s][q]));
+            }
+#pragma unroll
+        for (int t = 0; t < IS; ++t)
+#pragma unroll
+          for (int s = 0; s < JS; ++s)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v[t][s][q] += old[t][s][q];
       }
+      // Store order: the pieces of one row right after each other (with paired
+      // rhs fragments v[.][0][q] and v[.][1][q] are the two halves of 32
+      // contiguous bytes), then the neighbouring row of the other lhs fragment.
 #pragma unroll
-      for (int s = 0; s < JS; ++s)
+      for (int q = 0; q < 4; ++q)
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-          if (row_inside && (col_inside >> (4 * (j0 + s) + q) & 1))
-            *(stored_t*)(row_out + col_off[j0 + s][q]) = to_stored(v[s][q]);
+        for (int t = 0; t < IS; ++t)
+#pragma unroll
+          for (int s = 0; s < JS; ++s)
+            if (row_inside[t] && (col_inside >> (4 * (j0 + s) + q) & 1))
+              *(stored_t*)(row_out[t] + col_off[j0 + s][q]) = to_stored(v[t][s][q]);
       // Keep the fragments apart: hoisting all address arithmetic and
       // accumulator reads to the top costs more registers than there are.
       __builtin_amdgcn_sched_barrier(0);
