@@ -54,6 +54,7 @@ struct SkinnyArgs {
   int64_t out_stride0;  // elements
   int64_t tile_bytes;   // K * N0 * (bytes of an rhs row piece): one rhs tile row
   int32_t rows;         // M * M0
+  int32_t row0;         // first lhs row of this launch (the kernel covers rows row0 .. row0 + ROWS - 1)
   int32_t N, K;
   int32_t log2_M0, log2_N0;
   int32_t accumulate;
@@ -227,7 +228,7 @@ __global__ __launch_bounds__(256) void mmt4d_skinny_kernel(const SkinnyArgs a) {
   const uint8_t* lhs_row[ROWS];
 #pragma unroll
   for (int m = 0; m < ROWS; ++m) {
-    const int row = m < a.rows ? m : a.rows - 1;  // clamp: computed, not stored
+    const int row = a.row0 + m < a.rows ? a.row0 + m : a.rows - 1;  // clamp: computed, not stored
     lhs_row[m] = a.lhs + (int64_t)(row >> a.log2_M0) * a.lhs_stride_bytes + (row & (M0 - 1)) * LHS_G;
   }
 
@@ -276,12 +277,13 @@ __global__ __launch_bounds__(256) void mmt4d_skinny_kernel(const SkinnyArgs a) {
   }
   __syncthreads();
   const int t = threadIdx.x;
-  const int m = t >> a.log2_N0, j0 = t & (N0 - 1);
-  if (m < a.rows) {
-    acc_t sum = partial[0][m][j0];
-    sum += partial[1][m][j0];
-    sum += partial[2][m][j0];
-    sum += partial[3][m][j0];
+  const int slab_row = t >> a.log2_N0, j0 = t & (N0 - 1);
+  const int m = a.row0 + slab_row;
+  if (slab_row < ROWS && m < a.rows) {
+    acc_t sum = partial[0][slab_row][j0];
+    sum += partial[1][slab_row][j0];
+    sum += partial[2][slab_row][j0];
+    sum += partial[3][slab_row][j0];
     if constexpr (KIND == kI8I4) sum >>= 4;
     const int64_t index = (int64_t)(m >> a.log2_M0) * a.out_stride0 +
                           ((int64_t)blockIdx.x << (a.log2_M0 + a.log2_N0)) + ((m & (M0 - 1)) << a.log2_N0) + j0;
@@ -335,12 +337,19 @@ bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, int* piece_bytes,
   if (g != 2 && g != 4 && g != 8) return false;
   const int lm0 = log2_exact(a.M0), ln0 = log2_exact(a.N0);
   // A k step of the rhs must be whole 16-byte vectors.
-  if (lm0 < 0 || ln0 < 0 || a.M0 > 8 || a.N0 > 32 || a.N0 * g < 16) return false;
+  // Types that no matrix kernel takes (16-bit integers) may have any number of
+  // lhs rows: they are worked off eight at a time (launch_skinny), each slab
+  // streaming the rhs again. For everything else more than 8 rows belong to
+  // the block kernels.
+  const bool any_rows = *kind == kI16 || u4;
+  if (lm0 < 0 || ln0 < 0 || a.M0 > (any_rows ? 16 : 8) || a.N0 > 32 || a.N0 * g < 16) return false;
   *piece_bytes = g;
   if (probe_only) return a.M0 * lhs_g < 16 || *kind == kI16 || u4 || (i4 && a.K0 < 16);  // what no matrix kernel takes
   // 16x-scaled int4 accumulation must not overflow int32.
   if (i4 && (int64_t)a.K * a.K0 >= 131072) return false;
-  if (a.M * a.M0 > 8 || a.M <= 0 || a.K <= 0 || a.N <= 0 || a.N > 0x7FFFFFFF) return false;
+  if ((!any_rows && a.M * a.M0 > 8) || a.M * a.M0 > 0x7FFFFFFF || a.M <= 0 || a.K <= 0 || a.N <= 0 ||
+      a.N > 0x7FFFFFFF)
+    return false;
   if ((u4 || i4) && (a.rhs_stride0 & 1)) return false;
   const int64_t lhs_stride_bytes = a.lhs_stride0 * elem_bytes;
   const int64_t rhs_stride_bytes = (u4 || i4) ? a.rhs_stride0 / 2 : a.rhs_stride0 * elem_bytes;
@@ -353,6 +362,7 @@ bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, int* piece_bytes,
   s->out_stride0 = a.out_stride0;
   s->tile_bytes = a.K * a.N0 * g;
   s->rows = (int32_t)(a.M * a.M0);
+  s->row0 = 0;
   s->N = (int32_t)a.N;
   s->K = (int32_t)a.K;
   s->log2_M0 = lm0;
@@ -362,14 +372,21 @@ bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, int* piece_bytes,
 }
 
 template <int KIND, int G, bool NARROW>
-hipError_t launch_piece(const SkinnyArgs& s, hipStream_t stream) {
-  // Fewer lhs rows leave registers for more of the rhs stream in flight.
-  const dim3 grid((unsigned)s.N), block(256);
-  if (s.rows <= 1) hipLaunchKernelGGL((mmt4d_skinny_kernel<KIND, G, 1, 16, NARROW>), grid, block, 0, stream, s);
-  else if (s.rows <= 2) hipLaunchKernelGGL((mmt4d_skinny_kernel<KIND, G, 2, 16, NARROW>), grid, block, 0, stream, s);
-  else if (s.rows <= 4) hipLaunchKernelGGL((mmt4d_skinny_kernel<KIND, G, 4, 8, NARROW>), grid, block, 0, stream, s);
-  else hipLaunchKernelGGL((mmt4d_skinny_kernel<KIND, G, 8, 4, NARROW>), grid, block, 0, stream, s);
-  return hipGetLastError();
+hipError_t launch_piece(const SkinnyArgs& all_rows, hipStream_t stream) {
+  // Fewer lhs rows leave registers for more of the rhs stream in flight. More
+  // than 8 rows (types without a block kernel): one launch per slab of 8.
+  const dim3 grid((unsigned)all_rows.N), block(256);
+  SkinnyArgs s = all_rows;
+  for (s.row0 = 0; s.row0 < s.rows; s.row0 += 8) {
+    const int left = s.rows - s.row0;
+    if (left <= 1) hipLaunchKernelGGL((mmt4d_skinny_kernel<KIND, G, 1, 16, NARROW>), grid, block, 0, stream, s);
+    else if (left <= 2) hipLaunchKernelGGL((mmt4d_skinny_kernel<KIND, G, 2, 16, NARROW>), grid, block, 0, stream, s);
+    else if (left <= 4) hipLaunchKernelGGL((mmt4d_skinny_kernel<KIND, G, 4, 8, NARROW>), grid, block, 0, stream, s);
+    else hipLaunchKernelGGL((mmt4d_skinny_kernel<KIND, G, 8, 4, NARROW>), grid, block, 0, stream, s);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
 }
 
 template <int KIND, bool NARROW>

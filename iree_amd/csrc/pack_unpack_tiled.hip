@@ -903,6 +903,15 @@ hipError_t launch_pack(const PackArgs& original, hipStream_t stream, const char*
     a.out_size2 = 1;
     tr_inner = true;
   }
+  // The other way round for 4-byte elements: a tile one ROW tall stored
+  // inner-transposed ([T1][1]) is that row's T1 consecutive elements, i.e. the
+  // untransposed [1][T1]; as such its 16-byte vectors are whole pieces of a
+  // row in LDS instead of four separate elements.
+  if (tr_inner && a.out_size3 == 1 && a.elem_bytes == 4) {
+    a.out_size3 = a.out_size2;
+    a.out_size2 = 1;
+    tr_inner = false;
+  }
   if (!make_plan(a.in, a.out, a.in_stride0, a.in_stride1, a.out_stride0, a.in_size0, a.in_size1,
                  a.out_size0, a.out_size1, a.out_size2, a.out_size3, tr_inner, tr_outer,
                  a.elem_bytes, /*for_unpack=*/false, &plan))
@@ -930,14 +939,22 @@ hipError_t launch_pack(const PackArgs& original, hipStream_t stream, const char*
   return launch_plan<false>(plan, stream);
 }
 
-hipError_t launch_unpack(const UnpackArgs& a, hipStream_t stream, const char** name) {
+hipError_t launch_unpack(const UnpackArgs& original, hipStream_t stream, const char** name) {
   Plan plan;
-  const bool tr_inner = a.flags & IREE_UK_FLAG_UNPACK_TRANSPOSE_INNER;
+  UnpackArgs a = original;
+  bool tr_inner = a.flags & IREE_UK_FLAG_UNPACK_TRANSPOSE_INNER;
   const bool tr_outer = a.flags & IREE_UK_FLAG_UNPACK_TRANSPOSE_OUTER;
+  // A tile one row tall stored inner-transposed is the untransposed [1][T1]
+  // (see launch_pack).
+  if (tr_inner && a.in_size3 == 1) {
+    a.in_size3 = a.in_size2;
+    a.in_size2 = 1;
+    tr_inner = false;
+  }
   if (!make_plan(a.out, a.in, a.out_stride0, a.out_stride1, a.in_stride0, a.out_size0, a.out_size1,
                  a.in_size0, a.in_size1, a.in_size2, a.in_size3, tr_inner, tr_outer, a.elem_bytes,
                  /*for_unpack=*/true, &plan))
-    return launch_unpack_generic(a, stream, name);
+    return launch_unpack_generic(original, stream, name);
   plan.args.src = a.in;
   plan.args.dst = a.out;
   plan.args.padding_value = 0;

@@ -386,6 +386,30 @@ void mmt4d_impl(const iree_uk_mmt4d_params_t* p, Stager& stager) {
   a.M0 = p->M0; a.N0 = p->N0; a.K0 = p->K0;
   a.flags = p->flags;
 
+  // The int4 kernels carry 16x the sums in int32, which holds for a total depth
+  // below 131072. A deeper product is computed as a chain of calls over slices
+  // of K, every slice after the first accumulating onto the output (exact:
+  // int32 addition wraps the same way in any grouping).
+  const int64_t depth_limit = 131072;
+  if ((p->flags & IREE_UK_FLAG_MMT4D_TYPE_MASK) == IREE_UK_FLAG_MMT4D_TYPE_S8S4S32 && p->K0 > 0 &&
+      p->K * p->K0 >= depth_limit && select_mmt4d(a, /*probe_only=*/true)) {
+    // (A multiple of 8 k steps: whole 128-value steps of the matrix-vector kernel, whole chunks of the block kernels.)
+    int64_t slice = (depth_limit - 1) / p->K0;
+    if (slice > 8) slice &= ~(int64_t)7;
+    for (int64_t k = 0; k < p->K; k += slice) {
+      uk::Mmt4dArgs part = a;
+      part.K = p->K - k < slice ? p->K - k : slice;
+      part.lhs = a.lhs + k * p->M0 * p->K0;
+      part.rhs = a.rhs + k * p->N0 * p->K0 / 2;
+      if (k > 0) part.flags |= IREE_UK_FLAG_MMT4D_ACCUMULATE;
+      uk::Mmt4dLauncher launcher = select_mmt4d(part, /*probe_only=*/false);
+      if (!launcher) launcher = uk::launch_mmt4d_generic;
+      if (!launch_ok(launcher(part, stream, &tl_last_kernel), "mmt4d")) return;
+    }
+    finish(stream, s_out, out_region, s_lhs.host || s_rhs.host || s_out.host);
+    return;
+  }
+
   uk::Mmt4dLauncher launcher = select_mmt4d(a, /*probe_only=*/false);
   if (!launcher) launcher = uk::launch_mmt4d_generic;
   if (!launch_ok(launcher(a, stream, &tl_last_kernel), "mmt4d")) return;

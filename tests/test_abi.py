@@ -208,15 +208,16 @@ def test_mmt4d_info_reports_specialised_kernels():
                             (abi.MMT4D_TYPE_BF16BF16F32, 2, 16, 2), (abi.MMT4D_TYPE_BF16BF16BF16 | skip, 8, 8, 4),
                             (abi.MMT4D_TYPE_F32F32F32, 1, 16, 1), (abi.MMT4D_TYPE_F32F32F32, 16, 16, 1),
                             (abi.MMT4D_TYPE_S8S8S32, 8, 8, 8), (abi.MMT4D_TYPE_S8S8S32, 2, 8, 4),
-                            (abi.MMT4D_TYPE_S16S16S32, 1, 16, 2), (abi.MMT4D_TYPE_S16U4S32, 1, 32, 8),
+                            (abi.MMT4D_TYPE_S16S16S32, 1, 16, 2), (abi.MMT4D_TYPE_S16S16S32, 16, 16, 2), (abi.MMT4D_TYPE_S16U4S32, 1, 32, 8),
                             (abi.MMT4D_TYPE_S8S4S32, 4, 8, 8), (abi.MMT4D_TYPE_S8S4S32, 1, 8, 16)]:
         assert lib.iree_uk_mmt4d_info(m0, n0, k0, t, None) == 1, (hex(t), m0, n0, k0)
     assert lib.iree_uk_mmt4d_info(9, 6, 3, abi.MMT4D_TYPE_S8S8S32, None) == 0
     assert lib.iree_uk_mmt4d_info(8, 8, 4, 0x0B, None) == 0
-    # What only the generic kernel takes: one-byte row pieces, 16-bit integers in 16-row tiles, f16f16f16 with a
+    # What only the generic kernel takes: one-byte row pieces, s16s8s32 (no CPU target of the reference has a tile for
+    # it either), f16f16f16 with a
     # rounding after every k step.
     assert lib.iree_uk_mmt4d_info(8, 8, 1, abi.MMT4D_TYPE_S8S8S32, None) == 0
-    assert lib.iree_uk_mmt4d_info(16, 16, 2, abi.MMT4D_TYPE_S16S16S32, None) == 0
+    assert lib.iree_uk_mmt4d_info(16, 16, 2, abi.MMT4D_TYPE_S16S8S32, None) == 0
     assert lib.iree_uk_mmt4d_info(16, 16, 1, abi.MMT4D_TYPE_F16F16F16, None) == 0
 
 

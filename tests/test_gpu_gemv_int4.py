@@ -28,7 +28,7 @@ CASES = [
     (1, 16, 50, 20, 64, b"mmt4d_gemv"),
     (1, 16, 18, 3, 32, None),                 # K * K0 = 96: not a whole step
     (1, 16, 18, 8, 16, None),                 # 8-byte rhs row pieces
-    (1, 2, 18, 2048, 64, None),               # K * K0 = 131072: 16x-scaled sums could overflow
+    (1, 2, 18, 2048, 64, b"mmt4d_gemv"),      # K * K0 = 131072: 16x-scaled sums could overflow; chained over two slices of K
 ]
 
 

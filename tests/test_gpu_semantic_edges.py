@@ -111,3 +111,29 @@ def test_f16_subnormal_inputs_deviate_from_the_flushing_reference_by_at_most_the
     assert np.all(np.abs(got - flushed) <= bound + 1e-5 * rms)
     # ... and on this data that is far inside the tolerance stated for the float kernels.
     assert np.all(np.abs(got - flushed) <= tol)
+
+
+@pytest.mark.parametrize("M,N,M0", [(2, 3, 16), (1, 40, 1)])
+def test_int4_products_deeper_than_the_scaled_accumulators_hold(gpu_lib, oracle_lib, M, N, M0):
+    # The int4 kernels keep 16x the sums in int32, good for a total depth below
+    # 131072; a deeper product is chained over slices of K. Worst-case operands
+    # (-128 x -8 everywhere) so that an overflow of a slice would show.
+    N0, K0, K = 16, 32, 4100                      # depth 131200
+    flags = abi.MMT4D_TYPE_S8S4S32
+    lhs = synth.uniform_int8(51, 0, M * K * M0 * K0)
+    rhs = synth.uniform_int4_packed(51, 1, N * K * N0 * K0)
+    lhs[:K * M0 * K0] = -128                      # first lhs tile row: extreme values
+    rhs[:K * N0 * K0 // 2] = 0x88                 # first rhs panel: -8 in every nibble
+    init = (synth.bits64(51, 2, M * N * M0 * N0) & np.uint64(0xFFFF)).astype(np.int32)
+    for accumulate in (0, abi.MMT4D_ACCUMULATE):
+        want = init.copy()
+        oracle_lib.oracle_mmt4d_mt(C.byref(_params(lhs.ctypes.data, rhs.ctypes.data, want.ctypes.data, M, N, K, M0, N0,
+                                                   K0, flags | accumulate | abi.MMT4D_ALLOW_GENERIC_FALLBACK,
+                                                   K * M0 * K0, K * N0 * K0)), 8)
+        d_l, d_r = torch.from_numpy(lhs).cuda(), torch.from_numpy(rhs).cuda()
+        d_o = torch.from_numpy(init).cuda()
+        gpu_lib.iree_uk_mmt4d_p(C.byref(_params(d_l.data_ptr(), d_r.data_ptr(), d_o.data_ptr(), M, N, K, M0, N0, K0,
+                                                flags | accumulate, K * M0 * K0, K * N0 * K0)))
+        assert b"generic" not in gpu_lib.iree_uk_mi355x_last_kernel()
+        assert np.array_equal(d_o.cpu().numpy(), want), (M, N, accumulate)
+    assert want[0] == init[0] + 131200 * 1024    # (-128) * (-8) * depth on top of the initial value

@@ -119,9 +119,15 @@ def test_int4_weights_in_narrow_tiles(gpu_lib, M, M0, N0, K0):
              accumulate=True, seed=3)
 
 
-def test_sixteen_bit_integer_types_with_more_rows_stay_generic(gpu_lib):
-    run_s16_case(gpu_lib, False, 2, 9, 20, 8, 16, 2, True, "mmt4d_generic")
-    run_s16_case(gpu_lib, True, 1, 9, 20, 16, 32, 8, False, "mmt4d_generic")
+def test_sixteen_bit_integer_types_with_more_rows_are_worked_off_in_slabs(gpu_lib):
+    # No matrix kernel exists for them: any number of rows goes through this kernel eight rows at a time, also the
+    # 16-row tiles of the x86-64 VNNI target (s16s16s32 16x16x2, mmt4d_x86_64_tiles.inl:69,74).
+    run_s16_case(gpu_lib, False, 2, 9, 20, 8, 16, 2, True, "mmt4d_skinny")
+    run_s16_case(gpu_lib, False, 5, 33, 300, 16, 16, 2, False, "mmt4d_skinny", seed=4)      # 80 rows
+    run_s16_case(gpu_lib, False, 3, 7, 64, 16, 8, 2, True, "mmt4d_skinny", seed=5)          # 48 rows, 8-row rhs tiles
+    run_s16_case(gpu_lib, False, 13, 5, 64, 1, 16, 2, True, "mmt4d_skinny", seed=6)         # 13 rows: slabs of 8 + 5
+    run_s16_case(gpu_lib, True, 1, 9, 20, 16, 32, 8, False, "mmt4d_skinny", seed=7)
+    run_s16_case(gpu_lib, True, 21, 9, 40, 1, 32, 8, True, "mmt4d_skinny", seed=8)
 
 
 def test_more_rows_than_the_kernel_takes_fall_through(gpu_lib):
