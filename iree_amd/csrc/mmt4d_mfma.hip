@@ -59,6 +59,11 @@ bool make_plan(const Mmt4dArgs& a, bool probe_only, Plan* plan) {
     gather = 16;
   } else if (lhs_rb >= 16 && lhs_rb <= 64) {
     gather = 16;
+  } else if (lhs_rb == 1 && kind == kI8) {
+    // int8 K0 = 1 (the Arm baseline tiles Mx8x1): k-major operands, transposed
+    // on the way out of LDS; tiles of 8 or 16 rows, direct-to-LDS kernel only.
+    if (lm0 < 3 || ln0 < 3) return false;
+    gather = 1;
   } else if (lhs_rb == 4 || lhs_rb == 2 || lhs_rb == 8) {
     // 2 and 8 (e.g. the x86-64 int8 16x16x2 and f16 16x16x1 tiles, the Arm int8
     // 8x8x8 tiles) run on the direct-to-LDS kernel only: see below.
@@ -73,7 +78,7 @@ bool make_plan(const Mmt4dArgs& a, bool probe_only, Plan* plan) {
   if (probe_only) return true;
 
   // Alignment of every vector access the kernel makes.
-  const int lhs_align = gather == 4 ? 4 : 16;
+  const int lhs_align = gather == 4 ? 4 : 16;  // (also for 1-, 2- and 8-byte pieces: 16 bytes per lane)
   const int rhs_align = i4 ? 8 : lhs_align;
   const int64_t lhs_stride_bytes = a.lhs_stride0 * elem_bytes;
   const int64_t rhs_stride_bytes = i4 ? a.rhs_stride0 / 2 : a.rhs_stride0 * elem_bytes;
@@ -101,7 +106,7 @@ bool make_plan(const Mmt4dArgs& a, bool probe_only, Plan* plan) {
   m.log2_lhs_rb = llrb; m.log2_rhs_rb = lrrb;
   m.chunks = (int32_t)(((int64_t)a.K * lhs_rb + 63) / 64);
   m.accumulate = (a.flags & IREE_UK_FLAG_MMT4D_ACCUMULATE) ? 1 : 0;
-  if ((gather == 2 || gather == 8) && !mfma_direct_covers(m, gather, i4)) return false;
+  if ((gather == 1 || gather == 2 || gather == 8) && !mfma_direct_covers(m, gather, i4)) return false;
   return true;
 }
 

@@ -580,6 +580,17 @@ __device__ __forceinline__ void load_to_lds(uint32_t lds_off, uint32_t voff, con
                : "memory");
 }
 
+// 8 bytes per lane from LDS, transposed within each group of 16 lanes
+// (ds_read_b64_tr_b8): the 16 lanes' 8-byte chunks are taken as 8 rows of 16
+// bytes (chunks 2j and 2j + 1 make row j), and lane i of the group receives
+// byte i of every row. With a k-major operand ("16 matrix rows at k, then the
+// same rows at k + 1, ...") lane i thus gets 8 consecutive k of matrix row i.
+__device__ __forceinline__ uint2 lds_read_transposed(const uint8_t* p) {
+  typedef int v2i32 __attribute__((ext_vector_type(2)));
+  const v2i32 v = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i32*)(p));
+  return make_uint2((uint32_t)v.x, (uint32_t)v.y);
+}
+
 template <int N>
 __device__ __forceinline__ void wait_loads_but() {
   static_assert(N >= 0 && N <= 63, "vmcnt is a 6-bit counter");
@@ -703,6 +714,34 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
                                        a.rhs_stride_bytes, a.rhs_rb) +
                             ((16 * c) >> a.log2_rhs_rb) * rhs_kstep + ((16 * c) & (a.rhs_rb - 1)));
     }
+  } else if constexpr (G == 1) {
+    // One-byte row pieces (K0 = 1 int8: the operand is k-major, M0 bytes per k
+    // step). A load brings one group of 16 rows x 64 k steps = 1 KiB, group
+    // m = 4*t + w of the operand (fragment m >> 1), into slots 64*m .. 64*m + 63:
+    // 16-row tiles: lane l the 16 rows at k step l; 8-row tiles: lane l the 8
+    // rows of tile l & 1 of the group at k steps 2*(l >> 1) and + 1. Either
+    // way a k step's 16 rows lie within 32 bytes of LDS and the transposing
+    // read (lds_read_transposed) hands lane (r, h) 8 consecutive k of row r; two
+    // of them make a K-step's 16 bytes, in ascending k like every layout here.
+    auto piece_of = [&](int log2_t0, int t, int* row, int* k1) {
+      const int group = 4 * t + wave;
+      *row = 16 * group + (log2_t0 == 4 ? 0 : 8 * (lane & 1));
+      *k1 = log2_t0 == 4 ? lane : 2 * (lane >> 1);
+    };
+#pragma unroll
+    for (int t = 0; t < A_LOADS; ++t) {
+      int row, k1;
+      piece_of(a.log2_M0, t, &row, &k1);
+      a_off[t] = (uint32_t)(row_offset(first_row + row, total_rows - (1 << a.log2_M0), first_row, a.log2_M0,
+                                       a.lhs_stride_bytes, a.lhs_rb) + k1 * lhs_kstep);
+    }
+#pragma unroll
+    for (int t = 0; t < B_LOADS; ++t) {
+      int row, k1;
+      piece_of(a.log2_N0, t, &row, &k1);
+      b_off[t] = (uint32_t)(row_offset(first_col + row, total_cols - (1 << a.log2_N0), first_col, a.log2_N0,
+                                       a.rhs_stride_bytes, a.rhs_rb) + k1 * rhs_kstep);
+    }
   } else {
     constexpr int R = 16 / G;  // rows per 16-byte piece
     // Row group and k step of the chunk of this lane's piece in load t (the
@@ -785,6 +824,15 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
       return *(const uint32_t*)(first + (part >> 1) * 512 + 4 * (part & 1));
     }
   };
+  // G == 1: byte offset of lane (r, h)'s transposing reads inside a fragment's
+  // 2 KiB (two 16-row groups of 1 KiB, k-major): group r >> 4, k steps from 16*h,
+  // and the lane's chunk c = r & 15 of the 16 that one read transposes: the 8
+  // rows 8*(c & 1) .. + 7 at k step c >> 1.
+  auto transposed_lane_offset = [&](int log2_t0) -> int32_t {
+    const int c = lane & 15;
+    const int chunk = log2_t0 == 4 ? 8 * c : 32 * (c >> 2) + 16 * (c & 1) + 8 * ((c >> 1) & 1);
+    return 1024 * ((lane & 31) >> 4) + 256 * (lane >> 5) + chunk;
+  };
   // Fragment f of an operand at 16-byte slot `operand` of the ring, K-step kk.
   auto read_frag = [&](int operand, int f, int kk) -> uint4 {
     if (RHS_I4 && operand >= A_PIECES) {
@@ -794,6 +842,11 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
     if constexpr (G == 16) {
       if (!RHS_I4) return ring[operand + 128 * f + 32 * kk + 64 * ((lane & 31) >> 4) + 16 * (lane >> 5) + (lane & 15)];
       return ring[operand + 128 * f + 64 * kk + lane];
+    } else if constexpr (G == 1) {
+      const uint8_t* first = (const uint8_t*)(ring + operand) + 2048 * f + 512 * kk +
+                             transposed_lane_offset(operand >= A_PIECES ? a.log2_N0 : a.log2_M0);
+      const uint2 lo = lds_read_transposed(first), hi = lds_read_transposed(first + 128);
+      return make_uint4(lo.x, lo.y, hi.x, hi.y);
     } else {
       const uint8_t* first = (const uint8_t*)(ring + operand) + 1024 * (2 * f + kk) + G * lane;
       return make_uint4(gather_dword(first, 0), gather_dword(first, 1), gather_dword(first, 2), gather_dword(first, 3));
@@ -831,15 +884,18 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   constexpr bool ROWS16 = G == 16 && !RHS_I4;
   const uint8_t* ring_bytes =
       (const uint8_t*)ring + (ROWS16 ? 16 * (64 * ((lane & 31) >> 4) + 16 * (lane >> 5) + (lane & 15))
-                                     : (G == 16 ? 16 : G) * lane);
+                                     : (G == 1 ? 0 : (G == 16 ? 16 : G) * lane));
   // G == 2: lanes address dwords, not 16-bit elements. Paired: dword number
   // lane; unpaired: the dword that holds the lane's element (two lanes share
   // it), from which `own_half` then picks the low or the high half. (16-bit
   // reads that fill the halves of a register one after the other made these
   // tiles 1.8x slower than the 4-byte ones: the second read of a register has
   // to wait for the first.)
-  const int32_t pair_a_lane = G != 2 ? 0 : (PAIR_A ? 2 * lane : -2 * (lane & 1));
-  const int32_t pair_b_lane = G != 2 ? 0 : (PAIR_B ? 2 * lane : -2 * (lane & 1));
+  // (G == 1: the per-operand lane offset of the transposing reads instead.)
+  const int32_t pair_a_lane =
+      G == 1 ? transposed_lane_offset(a.log2_M0) : (G != 2 ? 0 : (PAIR_A ? 2 * lane : -2 * (lane & 1)));
+  const int32_t pair_b_lane =
+      G == 1 ? transposed_lane_offset(a.log2_N0) : (G != 2 ? 0 : (PAIR_B ? 2 * lane : -2 * (lane & 1)));
   const uint32_t own_half = (lane & 1) ? 0x07060302u : 0x05040100u;
   constexpr int KK16 = ROWS16 ? 32 : 64;
 
@@ -954,7 +1010,11 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
               dst = *(const uint4*)(src + (128 * frag + KK16 * kk) * 16);
             } else {
               const uint8_t* first = src + 1024 * (2 * frag + kk);
-              if constexpr (G == 2) {
+              if constexpr (G == 1) {
+                // One transposing read: 8 consecutive k of the lane's row.
+                const uint2 w = lds_read_transposed(src + 2048 * frag + 512 * kk + 128 * part);
+                if (part == 0) { dst.x = w.x; dst.y = w.y; } else { dst.z = w.x; dst.w = w.y; }
+              } else if constexpr (G == 2) {
                 // Elements 2*part and 2*part + 1 of the lane's eight, 128 bytes apart, each with its neighbour.
                 raw_pair[u] = make_uint2(*(const uint32_t*)(first + 256 * part), *(const uint32_t*)(first + 256 * part + 128));
                 (void)dst;
@@ -1308,6 +1368,10 @@ bool direct_covers(const MfmaArgs& m) {
   if (row_bytes % 64 != 0 && (RHS_I4 || row_bytes < 64)) return false;
   if (RHS_I4) return m.rhs_rb >= 16 && (uintptr_t)m.rhs % 16 == 0 && m.rhs_stride_bytes % 16 == 0;
   if (G == 16) return true;
+  // One-byte pieces: tiles of 8 or 16 rows (a 16-byte piece is one or two k steps of a whole tile).
+  if (G == 1)
+    return m.log2_M0 >= 3 && m.log2_N0 >= 3 && (uintptr_t)m.lhs % 16 == 0 && (uintptr_t)m.rhs % 16 == 0 &&
+           m.lhs_stride_bytes % 16 == 0 && m.rhs_stride_bytes % 16 == 0;
   // 16 / G rows of one k step make up a lane's 16 bytes: tiles at least that tall.
   return (G << m.log2_M0) >= 16 && (G << m.log2_N0) >= 16 && (uintptr_t)m.lhs % 16 == 0 &&
          (uintptr_t)m.rhs % 16 == 0 && m.lhs_stride_bytes % 16 == 0 && m.rhs_stride_bytes % 16 == 0;

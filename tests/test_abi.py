@@ -213,19 +213,23 @@ def test_mmt4d_info_reports_specialised_kernels():
         assert lib.iree_uk_mmt4d_info(m0, n0, k0, t, None) == 1, (hex(t), m0, n0, k0)
     assert lib.iree_uk_mmt4d_info(9, 6, 3, abi.MMT4D_TYPE_S8S8S32, None) == 0
     assert lib.iree_uk_mmt4d_info(8, 8, 4, 0x0B, None) == 0
-    # What only the generic kernel takes: one-byte row pieces, s16s8s32 (no CPU target of the reference has a tile for
+    # What only the generic kernel takes: one-byte row pieces in tiles less than 8 rows tall, s16s8s32 (no CPU target of the reference has a tile for
     # it either), f16f16f16 with a
     # rounding after every k step.
-    assert lib.iree_uk_mmt4d_info(8, 8, 1, abi.MMT4D_TYPE_S8S8S32, None) == 0
+    assert lib.iree_uk_mmt4d_info(4, 8, 1, abi.MMT4D_TYPE_S8S8S32, None) == 0
+    assert lib.iree_uk_mmt4d_info(8, 8, 1, abi.MMT4D_TYPE_S8S8S32, None) == 1   # k-major int8: transposing LDS reads
     assert lib.iree_uk_mmt4d_info(16, 16, 2, abi.MMT4D_TYPE_S16S8S32, None) == 0
     assert lib.iree_uk_mmt4d_info(16, 16, 1, abi.MMT4D_TYPE_F16F16F16, None) == 0
 
 
 def test_query_tile_sizes_roles_are_consistent():
-    from iree_amd import ukernel
+    def query(flags):
+        p, o = abi.QueryTileSizes2dParams(flags=flags), abi.QueryTileSizes2dOutParams()
+        library.load().iree_uk_query_tile_sizes_2d(C.byref(p), C.byref(o))
+        return o.tile_size0, o.tile_size1
     for op in (abi.QTS_OP_MATMUL_I8I8I32, abi.QTS_OP_MATMUL_F16F16F32, abi.QTS_OP_MATMUL_BF16BF16F32,
                abi.QTS_OP_MATMUL_F32F32F32):
-        m0, k0 = ukernel.query_tile_sizes_2d(op | abi.QTS_ROLE_LHS)
-        n0, k0r = ukernel.query_tile_sizes_2d(op | abi.QTS_ROLE_RHS)
+        m0, k0 = query(op | abi.QTS_ROLE_LHS)
+        n0, k0r = query(op | abi.QTS_ROLE_RHS)
         assert k0 == k0r
-        assert ukernel.query_tile_sizes_2d(op | abi.QTS_ROLE_RESULT) == (m0, n0)
+        assert query(op | abi.QTS_ROLE_RESULT) == (m0, n0)
