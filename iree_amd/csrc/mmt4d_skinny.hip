@@ -1,5 +1,5 @@
 // mmt4d for skinny left-hand sides in the narrow tile shapes that the
-// reference's CPU targets pick for them: at most 8 lhs rows in total (e.g.
+// reference's CPU targets pick for them: few lhs rows in total (e.g.
 // M0 = 1, 2, 4 with M = 1) and row pieces (K0 elements) of 2, 4 or 8 bytes:
 // the x86-64 1x16x2 int8 / bf16 and 1x16x1 f16 / f32 tiles, the Arm 1x8x4 and
 // 1x8x8 int8 tiles and their 2- and 4-row siblings (mmt4d_x86_64_tiles.inl,
@@ -33,7 +33,18 @@
 // a dword are isolated in the high nibbles of two dwords (int8 values 16 times
 // the weights) and multiplied with the even resp. odd lhs bytes of the k step,
 // which are gathered once per lhs piece; the sums are shifted right by 4 at
-// the end (exact; K * K0 < 131072 keeps 16x the sums inside int32).
+// the end (exact; K * K0 < 131072 keeps 16x the sums inside int32). The Arm
+// baseline tiles Mx16x2 have one byte per rhs row and k step: a lane's 16 bytes
+// are 16 rows, and each row's two weights (x16, as above) are put beside each
+// other in a dword for one v_dot4_i32_i8 with the lhs pair.
+// And s16s8s32, for which the reference has the generic tile only
+// (mmt4d_tile_generic.c:145-176): the rhs bytes are sign-extended to 16-bit
+// pairs (v_perm_b32 with its sign-byte selectors) for v_dot2_i32_i16.
+//
+// More than 8 lhs rows are worked off in slabs of 8, each streaming the rhs
+// again: what the block kernels can load they do faster (the caller prefers
+// them), what they cannot is still far better off here than with one thread
+// per output element.
 #include "uk_device.h"
 #include "uk_internal.h"
 
@@ -44,7 +55,7 @@ typedef int v4i32 __attribute__((ext_vector_type(4)));
 typedef _Float16 v2f16 __attribute__((ext_vector_type(2)));
 typedef short v2i16 __attribute__((ext_vector_type(2)));
 
-enum Kind { kI8 = 0, kF16 = 1, kBF16 = 2, kF32 = 3, kI16 = 4, kI16U4 = 5, kI8I4 = 6 };
+enum Kind { kI8 = 0, kF16 = 1, kBF16 = 2, kF32 = 3, kI16 = 4, kI16U4 = 5, kI8I4 = 6, kI16I8 = 7 };
 
 struct SkinnyArgs {
   const uint8_t* lhs;
@@ -65,12 +76,14 @@ template <> struct Acc<kI8> { typedef int32_t type; };
 template <> struct Acc<kI16> { typedef int32_t type; };
 template <> struct Acc<kI16U4> { typedef int32_t type; };
 template <> struct Acc<kI8I4> { typedef int32_t type; };
+template <> struct Acc<kI16I8> { typedef int32_t type; };
 // The lhs piece of one k step in registers. Same bytes as an rhs piece (G, zero-extended to two dwords), except:
 // s16u4s32: 8 values of 16 bits against 8 nibbles; s8s4s32: 8 or 16 bytes against as many nibbles, kept as one
-// dword of the even and one of the odd bytes per 8.
+// dword of the even and one of the odd bytes per 8 (2 bytes as they are); s16s8s32: twice the bytes of the rhs piece.
 template <int KIND> struct LhsPiece { typedef uint2 type; };
 template <> struct LhsPiece<kI16U4> { typedef uint4 type; };
 template <> struct LhsPiece<kI8I4> { typedef uint4 type; };
+template <> struct LhsPiece<kI16I8> { typedef uint4 type; };
 
 __device__ __forceinline__ int32_t dot2_i16(uint32_t a, uint32_t b, int32_t c) {
   return __builtin_amdgcn_sdot2(__builtin_bit_cast(v2i16, a), __builtin_bit_cast(v2i16, b), c, false);
@@ -84,6 +97,13 @@ __device__ __forceinline__ float f16_hi(uint32_t w) { return (float)__builtin_bi
 template <int KIND, int G>
 __device__ __forceinline__ typename LhsPiece<KIND>::type load_lhs_piece(const uint8_t* p) {
   if constexpr (KIND == kI16U4) return *(const uint4*)p;
+  else if constexpr (KIND == kI16I8) {
+    if constexpr (G == 2) return make_uint4(*(const uint32_t*)p, 0, 0, 0);
+    else if constexpr (G == 4) {
+      const uint2 half = *(const uint2*)p;
+      return make_uint4(half.x, half.y, 0, 0);
+    } else return *(const uint4*)p;
+  } else if constexpr (KIND == kI8I4 && G == 1) return make_uint4(*(const uint16_t*)p, 0, 0, 0);
   else if constexpr (KIND == kI8I4) {
     uint4 raw = make_uint4(0, 0, 0, 0);
     if constexpr (G == 4) {
@@ -104,7 +124,35 @@ template <int KIND, int G>
 __device__ __forceinline__ void multiply_piece(const uint4 v, const typename LhsPiece<KIND>::type l,
                                                typename Acc<KIND>::type* acc) {
   const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-  if constexpr (KIND == kI8I4) {
+  if constexpr (KIND == kI8I4 && G == 1) {
+    // 16 rows of two nibbles each against the lhs pair in the low half of l.x.
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const uint32_t evens = (w[d] << 4) & 0xF0F0F0F0u, odds = w[d] & 0xF0F0F0F0u;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        // byte 0: row r of `evens`, byte 1: row r of `odds`, zeros above
+        const uint32_t pair = __builtin_amdgcn_perm(odds, evens, 0x0C0C0400u + 0x0101u * r);
+        acc[4 * d + r] = __builtin_amdgcn_sdot4((int)pair, (int)l.x, acc[4 * d + r], false);
+      }
+    }
+  } else if constexpr (KIND == kI16I8) {
+    const uint32_t lhs[4] = {l.x, l.y, l.z, l.w};
+    // The four bytes of a dword as two pairs of 16-bit values. The selectors 8..11 of
+    // v_perm_b32 give the sign of bytes 1, 3 (second operand) and 5, 7 (first operand)
+    // as 0x00 or 0xFF; the dword shifted up by a byte has bytes 0 and 2 at 5 and 7.
+    uint32_t pairs[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      pairs[2 * i] = __builtin_amdgcn_perm(w[i] << 8, w[i], 0x08010A00u);
+      pairs[2 * i + 1] = __builtin_amdgcn_perm(w[i] << 8, w[i], 0x09030B02u);
+    }
+    constexpr int PPR = G / 2;  // pairs per row piece
+#pragma unroll
+    for (int r = 0; r < 16 / G; ++r)
+#pragma unroll
+      for (int q = 0; q < PPR; ++q) acc[r] = dot2_i16(pairs[r * PPR + q], lhs[q], acc[r]);
+  } else if constexpr (KIND == kI8I4) {
     static_assert(G == 4 || G == 8, "8 or 16 nibbles per row piece");
     const uint32_t lhs[4] = {l.x, l.y, l.z, l.w};
 #pragma unroll
@@ -218,10 +266,10 @@ __global__ __launch_bounds__(256) void mmt4d_skinny_kernel(const SkinnyArgs a) {
   const int32_t M0 = 1 << a.log2_M0, N0 = 1 << a.log2_N0;
   // One k step of the rhs is N0 * G bytes = `lanes_per_kstep` lanes; a block of
   // 1 KiB holds whole k steps, so a lane keeps its rows from block to block.
-  const int log2_kstep_bytes = a.log2_N0 + (G == 2 ? 1 : (G == 4 ? 2 : 3));
+  const int log2_kstep_bytes = a.log2_N0 + (G == 1 ? 0 : (G == 2 ? 1 : (G == 4 ? 2 : 3)));
   const int log2_lanes_per_kstep = log2_kstep_bytes - 4;
   const int32_t kstep_in_block = lane >> log2_lanes_per_kstep;
-  constexpr int LHS_G = KIND == kI16U4 ? 16 : (KIND == kI8I4 ? 2 * G : G);  // bytes of an lhs row piece
+  constexpr int LHS_G = KIND == kI16U4 ? 16 : (KIND == kI8I4 || KIND == kI16I8 ? 2 * G : G);  // bytes of an lhs row piece
   const int32_t lhs_kstep_bytes = LHS_G << a.log2_M0;
 
   const uint8_t* rhs_tile = a.rhs + (int64_t)blockIdx.x * a.rhs_stride_bytes;
@@ -319,6 +367,7 @@ bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, int* piece_bytes,
     case IREE_UK_FLAG_MMT4D_TYPE_S16S16S32: *kind = kI16; elem_bytes = 2; break;
     case IREE_UK_FLAG_MMT4D_TYPE_S16U4S32: *kind = kI16U4; elem_bytes = 2; break;
     case IREE_UK_FLAG_MMT4D_TYPE_S8S4S32: *kind = kI8I4; elem_bytes = 1; break;
+    case IREE_UK_FLAG_MMT4D_TYPE_S16S8S32: *kind = kI16I8; elem_bytes = 2; break;
     case IREE_UK_FLAG_MMT4D_TYPE_F16F16F16:
       if (!skip_roundings) return false;
       *kind = kF16; elem_bytes = 2; *narrow = true;
@@ -329,30 +378,24 @@ bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, int* piece_bytes,
       break;
     default: return false;
   }
-  const bool u4 = *kind == kI16U4, i4 = *kind == kI8I4;
+  const bool u4 = *kind == kI16U4, i4 = *kind == kI8I4, i16i8 = *kind == kI16I8;
   if (u4 && a.K0 != 8) return false;
-  if (i4 && a.K0 != 8 && a.K0 != 16) return false;
-  const int g = u4 ? 4 : (i4 ? a.K0 / 2 : a.K0 * elem_bytes);  // bytes of an rhs row piece
-  const int lhs_g = u4 ? 16 : (i4 ? a.K0 : g);
-  if (g != 2 && g != 4 && g != 8) return false;
+  if (i4 && a.K0 != 2 && a.K0 != 8 && a.K0 != 16) return false;
+  const int g = u4 ? 4 : (i4 ? a.K0 / 2 : (i16i8 ? a.K0 : a.K0 * elem_bytes));  // bytes of an rhs row piece
+  const int lhs_g = u4 ? 16 : (i4 ? a.K0 : (i16i8 ? 2 * a.K0 : g));
+  if (g != 2 && g != 4 && g != 8 && !(i4 && g == 1)) return false;
   const int lm0 = log2_exact(a.M0), ln0 = log2_exact(a.N0);
   // A k step of the rhs must be whole 16-byte vectors.
-  // Types that no matrix kernel takes (16-bit integers) may have any number of
-  // lhs rows: they are worked off eight at a time (launch_skinny), each slab
-  // streaming the rhs again. For everything else more than 8 rows belong to
-  // the block kernels.
-  const bool any_rows = *kind == kI16 || u4;
-  if (lm0 < 0 || ln0 < 0 || a.M0 > (any_rows ? 16 : 8) || a.N0 > 32 || a.N0 * g < 16) return false;
+  if (lm0 < 0 || ln0 < 0 || a.M0 > 16 || a.N0 > 32 || a.N0 * g < 16) return false;
   *piece_bytes = g;
-  if (probe_only) return a.M0 * lhs_g < 16 || *kind == kI16 || u4 || (i4 && a.K0 < 16);  // what no matrix kernel takes
+  // What no matrix kernel takes.
+  if (probe_only) return a.M0 * lhs_g < 16 || *kind == kI16 || u4 || i16i8 || (i4 && a.K0 < 16);
   // 16x-scaled int4 accumulation must not overflow int32.
   if (i4 && (int64_t)a.K * a.K0 >= 131072) return false;
-  if ((!any_rows && a.M * a.M0 > 8) || a.M * a.M0 > 0x7FFFFFFF || a.M <= 0 || a.K <= 0 || a.N <= 0 ||
-      a.N > 0x7FFFFFFF)
-    return false;
+  if (a.M * a.M0 > 0x7FFFFFFF || a.M <= 0 || a.K <= 0 || a.N <= 0 || a.N > 0x7FFFFFFF) return false;
   if ((u4 || i4) && (a.rhs_stride0 & 1)) return false;
   const int64_t lhs_stride_bytes = a.lhs_stride0 * elem_bytes;
-  const int64_t rhs_stride_bytes = (u4 || i4) ? a.rhs_stride0 / 2 : a.rhs_stride0 * elem_bytes;
+  const int64_t rhs_stride_bytes = (u4 || i4) ? a.rhs_stride0 / 2 : (i16i8 ? a.rhs_stride0 : a.rhs_stride0 * elem_bytes);
   if ((uintptr_t)a.rhs % 16 || (a.N > 1 && rhs_stride_bytes % 16)) return false;
   if ((uintptr_t)a.lhs % lhs_g || (a.M > 1 && lhs_stride_bytes % lhs_g)) return false;
   if ((uintptr_t)a.out % (*narrow ? 2 : 4)) return false;
@@ -374,7 +417,7 @@ bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, int* piece_bytes,
 template <int KIND, int G, bool NARROW>
 hipError_t launch_piece(const SkinnyArgs& all_rows, hipStream_t stream) {
   // Fewer lhs rows leave registers for more of the rhs stream in flight. More
-  // than 8 rows (types without a block kernel): one launch per slab of 8.
+  // than 8 rows: one launch per slab of 8.
   const dim3 grid((unsigned)all_rows.N), block(256);
   SkinnyArgs s = all_rows;
   for (s.row0 = 0; s.row0 < s.rows; s.row0 += 8) {
@@ -412,7 +455,9 @@ hipError_t launch_skinny(const Mmt4dArgs& a, hipStream_t stream, const char** na
     case kI16: return launch_kind<kI16, false>(s, piece_bytes, stream);
     case kI16U4: return launch_piece<kI16U4, 4, false>(s, stream);
     case kI8I4:
+      if (piece_bytes == 1) return launch_piece<kI8I4, 1, false>(s, stream);
       return piece_bytes == 4 ? launch_piece<kI8I4, 4, false>(s, stream) : launch_piece<kI8I4, 8, false>(s, stream);
+    case kI16I8: return launch_kind<kI16I8, false>(s, piece_bytes, stream);
     default: return launch_kind<kF32, false>(s, piece_bytes, stream);
   }
 }

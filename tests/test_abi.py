@@ -209,16 +209,17 @@ def test_mmt4d_info_reports_specialised_kernels():
                             (abi.MMT4D_TYPE_F32F32F32, 1, 16, 1), (abi.MMT4D_TYPE_F32F32F32, 16, 16, 1),
                             (abi.MMT4D_TYPE_S8S8S32, 8, 8, 8), (abi.MMT4D_TYPE_S8S8S32, 2, 8, 4),
                             (abi.MMT4D_TYPE_S16S16S32, 1, 16, 2), (abi.MMT4D_TYPE_S16S16S32, 16, 16, 2), (abi.MMT4D_TYPE_S16U4S32, 1, 32, 8),
-                            (abi.MMT4D_TYPE_S8S4S32, 4, 8, 8), (abi.MMT4D_TYPE_S8S4S32, 1, 8, 16)]:
+                            (abi.MMT4D_TYPE_S8S4S32, 4, 8, 8), (abi.MMT4D_TYPE_S8S4S32, 1, 8, 16),
+                            (abi.MMT4D_TYPE_S8S4S32, 4, 16, 2), (abi.MMT4D_TYPE_S16S8S32, 16, 16, 2),
+                            (abi.MMT4D_TYPE_S16S8S32, 1, 8, 8)]:
         assert lib.iree_uk_mmt4d_info(m0, n0, k0, t, None) == 1, (hex(t), m0, n0, k0)
     assert lib.iree_uk_mmt4d_info(9, 6, 3, abi.MMT4D_TYPE_S8S8S32, None) == 0
     assert lib.iree_uk_mmt4d_info(8, 8, 4, 0x0B, None) == 0
-    # What only the generic kernel takes: one-byte row pieces in tiles less than 8 rows tall, s16s8s32 (no CPU target of the reference has a tile for
-    # it either), f16f16f16 with a
-    # rounding after every k step.
+    # What only the generic kernel takes: one-byte row pieces in tiles less than 8 rows tall, tile sizes that are
+    # not powers of two (the reference tests s16s8s32 on 7x5x6), f16f16f16 with a rounding after every k step.
     assert lib.iree_uk_mmt4d_info(4, 8, 1, abi.MMT4D_TYPE_S8S8S32, None) == 0
     assert lib.iree_uk_mmt4d_info(8, 8, 1, abi.MMT4D_TYPE_S8S8S32, None) == 1   # k-major int8: transposing LDS reads
-    assert lib.iree_uk_mmt4d_info(16, 16, 2, abi.MMT4D_TYPE_S16S8S32, None) == 0
+    assert lib.iree_uk_mmt4d_info(7, 5, 6, abi.MMT4D_TYPE_S16S8S32, None) == 0
     assert lib.iree_uk_mmt4d_info(16, 16, 1, abi.MMT4D_TYPE_F16F16F16, None) == 0
 
 

@@ -73,10 +73,14 @@ def test_eight_row_tiles_a_matrix_kernel_can_load_go_there(gpu_lib):
 
 
 def run_s16_case(gpu_lib, u4, M, N, K, M0, N0, K0, accumulate, expect_kernel, seed=0):
-    """s16s16s32 or s16u4s32 against an exact float64 product (values small enough that no int32 sum wraps)."""
+    """s16s16s32, s16u4s32 (u4 True) or s16s8s32 (u4 "s8") against an exact float64 product (values small enough
+    that no int32 sum wraps)."""
     g = torch.Generator(device="cuda").manual_seed(seed)
     lhs = torch.randint(-300, 301, (M * K * M0 * K0,), dtype=torch.int16, device="cuda", generator=g)
-    if u4:
+    if u4 == "s8":
+        rhs = torch.randint(-128, 128, (N * K * N0 * K0,), dtype=torch.int8, device="cuda", generator=g)
+        b = rhs.view(N, K, N0, K0)
+    elif u4:
         packed = torch.randint(0, 256, (N * K * N0 * K0 // 2,), dtype=torch.uint8, device="cuda", generator=g)
         b = torch.stack([packed & 0xF, packed >> 4], dim=-1).reshape(N, K, N0, K0)  # element 2j in the low nibble of byte j
         rhs = packed
@@ -85,7 +89,8 @@ def run_s16_case(gpu_lib, u4, M, N, K, M0, N0, K0, accumulate, expect_kernel, se
         b = rhs.view(N, K, N0, K0)
     out = torch.randint(-1000, 1000, (M * N * M0 * N0,), dtype=torch.int32, device="cuda", generator=g)
     before = out.clone()
-    flags = (abi.MMT4D_TYPE_S16U4S32 if u4 else abi.MMT4D_TYPE_S16S16S32) | (abi.MMT4D_ACCUMULATE if accumulate else 0)
+    kind = abi.MMT4D_TYPE_S16S8S32 if u4 == "s8" else (abi.MMT4D_TYPE_S16U4S32 if u4 else abi.MMT4D_TYPE_S16S16S32)
+    flags = kind | (abi.MMT4D_ACCUMULATE if accumulate else 0)
     p = mm_params(lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), M, N, K, M0, N0, K0, flags)
     gpu_lib.iree_uk_mmt4d_p(C.byref(p))
     assert gpu_lib.iree_uk_mi355x_last_kernel() == expect_kernel.encode()
@@ -107,9 +112,41 @@ def test_sixteen_bit_integer_types(gpu_lib, u4, M, M0, N0, K0):
         run_s16_case(gpu_lib, u4, M, 23 + n, K, M0, N0, K0, bool(n & 1), "mmt4d_skinny", seed=K + M0)
 
 
-# int4 weights in the Arm tiles (s8s4s32 Mx8x8 with dot products, Mx8x16 with i8mm; mmt4d_arm_64_tiles.inl).
+# s16s8s32: the reference has the generic tile function only (mmt4d_tile_generic.c:145-176, tested on 7x5x6 tiles,
+# tools/mmt4d_test.c:550); power-of-two tiles with 2, 4 or 8 rhs bytes per k step run here, any number of rows.
+@pytest.mark.parametrize("M,M0,N0,K0", [(1, 1, 16, 2), (1, 4, 8, 2), (3, 2, 16, 2), (1, 1, 8, 4), (1, 8, 4, 4), (2, 4, 16, 4),
+                                        (1, 1, 2, 8), (1, 2, 8, 8), (5, 4, 4, 8), (2, 16, 16, 2)])
+def test_sixteen_bit_lhs_eight_bit_rhs(gpu_lib, M, M0, N0, K0):
+    for n, K in enumerate((1, 50, 1100)):
+        run_s16_case(gpu_lib, "s8", M, 23 + n, K, M0, N0, K0, bool(n & 1), "mmt4d_skinny", seed=K + M0 + K0)
+
+
+def test_sixteen_bit_lhs_eight_bit_rhs_extreme_values(gpu_lib, oracle_lib):
+    # -32768 x -128 and 32767 x -128 in every position: the widening of the rhs bytes must keep their sign, the sums
+    # wrap in int32 exactly as the reference's (mmt4d_tile_generic.c:145-176 accumulates in int32).
+    import numpy as np
+    M0, N0, K0, N, K = 4, 8, 4, 3, 600
+    lhs = np.full(K * M0 * K0, -32768, np.int16)
+    lhs[1::2] = 32767
+    rhs = np.full(N * K * N0 * K0, -128, np.int8)
+    rhs[::3] = 127
+    rhs[1::7] = -1
+    want = np.zeros(N * M0 * N0, np.int32)
+    flags = abi.MMT4D_TYPE_S16S8S32
+    oracle_lib.oracle_mmt4d(C.byref(mm_params(lhs.ctypes.data, rhs.ctypes.data, want.ctypes.data, 1, N, K, M0, N0, K0,
+                                              flags | abi.MMT4D_ALLOW_GENERIC_FALLBACK)))
+    d_l, d_r = torch.from_numpy(lhs).cuda(), torch.from_numpy(rhs).cuda()
+    d_o = torch.zeros(want.size, dtype=torch.int32, device="cuda")
+    gpu_lib.iree_uk_mmt4d_p(C.byref(mm_params(d_l.data_ptr(), d_r.data_ptr(), d_o.data_ptr(), 1, N, K, M0, N0, K0, flags)))
+    assert gpu_lib.iree_uk_mi355x_last_kernel() == b"mmt4d_skinny"
+    assert np.array_equal(d_o.cpu().numpy(), want)
+
+
+# int4 weights in the Arm tiles (s8s4s32 Mx16x2 baseline, Mx8x8 with dot products, Mx8x16 with i8mm;
+# mmt4d_arm_64_tiles.inl:50-59).
 @pytest.mark.parametrize("M,M0,N0,K0", [(1, 1, 8, 8), (1, 2, 8, 8), (1, 4, 8, 8), (1, 8, 8, 8), (1, 1, 8, 16), (1, 4, 8, 16),
-                                        (3, 1, 16, 16), (2, 2, 4, 8)])
+                                        (3, 1, 16, 16), (2, 2, 4, 8), (1, 1, 16, 2), (1, 2, 16, 2), (1, 4, 16, 2),
+                                        (3, 4, 16, 2), (1, 1, 32, 2), (3, 8, 8, 8)])
 def test_int4_weights_in_narrow_tiles(gpu_lib, M, M0, N0, K0):
     S8S4 = abi.MMT4D_TYPE_S8S4S32
     for n, K in enumerate((1, 33, 700)):
@@ -130,8 +167,9 @@ def test_sixteen_bit_integer_types_with_more_rows_are_worked_off_in_slabs(gpu_li
     run_s16_case(gpu_lib, True, 21, 9, 40, 1, 32, 8, True, "mmt4d_skinny", seed=8)
 
 
-def test_more_rows_than_the_kernel_takes_fall_through(gpu_lib):
-    # 9 rows of 1x16x2 int8 tiles: no matrix kernel loads such an lhs either; the generic kernel, still exact.
-    run_case(gpu_lib, S8, 9, 20, 40, 1, 16, 2, "mmt4d_generic", accumulate=True)
-    # rhs tile rows that are not 16-byte aligned
+def test_more_rows_than_one_slab_and_what_falls_through(gpu_lib):
+    # 9 rows of 1x16x2 int8 tiles: no matrix kernel loads such an lhs; two slabs (8 + 1 rows) here.
+    run_case(gpu_lib, S8, 9, 20, 40, 1, 16, 2, "mmt4d_skinny", accumulate=True)
+    run_case(gpu_lib, F32, 19, 20, 40, 1, 8, 1, "mmt4d_skinny")
+    # rhs tile rows that are not 16-byte aligned: the generic kernel, still exact
     run_case(gpu_lib, S8, 1, 20, 40, 1, 16, 2, "mmt4d_generic", rhs_pad=2)
