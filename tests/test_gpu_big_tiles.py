@@ -184,9 +184,9 @@ def test_two_byte_row_pieces_on_every_block_tile(gpu_lib, flags, M0, N0, K0, K):
 
 
 def test_narrow_row_pieces_fall_back_when_the_direct_kernel_cannot_run(gpu_lib):
-    # Less than one 64-byte chunk of K, or rows not 16-byte aligned: the generic kernel, still exact.
-    run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, 9, 11, 31, 16, 16, 2, "mmt4d_generic", accumulate=True)
-    run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, 9, 11, 32, 16, 16, 2, "mmt4d_generic", lhs_pad=4)
+    # Less than one 64-byte chunk of K, or rows not 16-byte aligned: the skinny kernel's 8-row slabs, still exact.
+    run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, 9, 11, 31, 16, 16, 2, "mmt4d_skinny", accumulate=True)
+    run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, 9, 11, 32, 16, 16, 2, "mmt4d_skinny", lhs_pad=4)
     run_case(gpu_lib, abi.MMT4D_TYPE_S8S8S32, 9, 11, 33, 16, 16, 2, "mmt4d_mfma_64x64", accumulate=True)
 
 
