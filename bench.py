@@ -238,6 +238,21 @@ def _also(torch, lib, abi, synth, steps, warmup):
         del va, vb
     except Exception as exc:  # not every torch build has it
         res["vendor_library_int8_gemm_4096_for_comparison"] = {"unavailable": str(exc)[:200]}
+    # The same for the f16 configuration's operands (f16 output there, f32 here).
+    try:
+        ha = f16_operand(3, 0, n, 1.0 / 64).view(torch.float16).view(4096, 4096)
+        hb = f16_operand(3, 1, n, 1.0 / 64).view(torch.float16).view(4096, 4096)
+        best = None
+        for operand in (hb, hb.t()):
+            ms, _ = _time_launches(torch, lambda: torch.matmul(ha, operand), steps, warmup)
+            best = ms if best is None else min(best, ms)
+        res["vendor_library_f16_gemm_4096_for_comparison"] = {
+            "what": "torch.matmul on f16 (f16 result, no accumulate input), best of B and B^T layouts",
+            "ms": round(best, 5), "value": round(2.0 * 4096 ** 3 / best / 1e9, 1), "unit": "TFLOP/s",
+            "frac_of_peak": round(2.0 * 4096 ** 3 / best / 1e9 / PEAK_F16_TFLOPS, 4)}
+        del ha, hb
+    except Exception as exc:
+        res["vendor_library_f16_gemm_4096_for_comparison"] = {"unavailable": str(exc)[:200]}
     res["e2e_pack_mmt4d_unpack_s8s8s32_4096"] = _e2e_chain(torch, lib, abi, synth, steps, warmup)
     # What the matrix pipe sustains on this device, measured by the
     # benchmark's probe (a helper library of its own): the 256x256 kernel's inner-loop instruction mix with no
@@ -465,6 +480,21 @@ def _also(torch, lib, abi, synth, steps, warmup):
     timed_pair("unpack_f32_512x8190x16x1_to_8191x8190", unpack_params, 2 * R * Cc * 4)
     torch.cuda.synchronize()
     res["pack_unpack_round_trip_bit_exact"] = bool(all(torch.equal(src[i], back[i]) for i in range(2)))
+    # What this device does on the same bytes with no rearrangement at all: the
+    # framework's device-to-device copy of the [8191, 8190] f32 matrix, same two
+    # buffer sets rotated. A ceiling to read the pack / unpack rows against, not a
+    # result of this library.
+    copy_state = {"i": 0}
+
+    def copy_step():
+        i = copy_state["i"] & 1
+        back[i].copy_(src[i])
+        copy_state["i"] += 1
+    ms, _ = _time_launches(torch, copy_step, max(steps, 6), warmup)
+    res["plain_device_copy_f32_8191x8190_for_comparison"] = {
+        "what": "torch.Tensor.copy_ of the same matrix (read + write counted)", "ms": round(ms, 5),
+        "value": round(2 * R * Cc * 4 / ms / 1e6, 1), "unit": "GB/s",
+        "frac_of_peak": round(2 * R * Cc * 4 / ms / 1e6 / PEAK_HBM_GBS, 4)}
     del src, packed, back
 
     # int8 operands of a 16384^3 matmul into the layouts of the 16x16x64 tile:
