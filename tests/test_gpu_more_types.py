@@ -145,3 +145,59 @@ def test_f32f32f32_4096_cubed_against_fp64_row_sample(gpu_lib):
     col_ref = a.double().sum(dim=0) @ b.double().t()
     col_got = out.double().sum(dim=0)
     assert bool(((col_got - col_ref).abs() <= 1e-3 * col_ref.abs().max()).all())
+
+
+def _operand_values(kind, count, seed):
+    """`count` finite, normal, nonzero 16-bit floats (as bit patterns) whose pairwise products cover what the final
+    rounding distinguishes: every result exponent from far below the output's range to overflow, exact ties (a
+    mantissa of 1.5 against odd multiples of the last place), values one place either side of a tie, all-ones
+    mantissas that carry into the exponent, both signs."""
+    ebits, mbits = (5, 10) if kind == "f16" else (8, 7)
+    bias = (1 << (ebits - 1)) - 1
+    rng = np.random.default_rng(seed)
+    mantissas = [0, 1 << (mbits - 1), (1 << mbits) - 1, 1, 3, (1 << (mbits - 1)) + 1, (1 << mbits) - 2]
+    out = []
+    for n in range(count):
+        # Exponent fields of normal numbers only. f16: all 30 of them; bf16: every other one, odd ones in one
+        # operand and even ones in the other, so that the products run from far below f32's range to beyond it.
+        e = 1 + (n * 7 + seed) % 30 if kind == "f16" else seed + 2 * (n % 127)
+        m = mantissas[n % len(mantissas)] if n % 3 else int(rng.integers(0, 1 << mbits))
+        sign = (n >> 2) & 1
+        out.append((sign << 15) | (e << mbits) | m)
+    assert bias > 0
+    return np.array(out, dtype=np.uint16)
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("K0", [16, 1])
+def test_16bit_output_rounding_matches_the_reference_on_every_exponent_and_on_ties(gpu_lib, oracle_lib, kind, K0):
+    # One product per output element (K = 1, the other K0 - 1 positions hold +0 in the lhs), so the f32 value that is
+    # rounded is exact and identical on both sides and the comparison pins the rounding itself (common.h:701-770),
+    # bit for bit: results below the output's exponent range (zero), in the lowest in-range exponent (exponent
+    # field 0 with mantissa bits), ties to even, carries into the exponent and to infinity, f16 products beyond 65504.
+    M, N, K, M0, N0 = 8, 8, 1, 16, 16
+    base = abi.MMT4D_TYPE_F16F16F16 if kind == "f16" else abi.MMT4D_TYPE_BF16BF16BF16
+    a = _operand_values(kind, M * M0, 1)
+    b = _operand_values(kind, N * N0, 2)
+    lhs = np.zeros((M, K, M0, K0), np.uint16)
+    rhs = np.full((N, K, N0, K0), 0x3C00 if kind == "f16" else 0x3F80, np.uint16)   # 1.0 in the unused positions
+    lhs[:, 0, :, 0] = a.reshape(M, M0)
+    rhs[:, 0, :, 0] = b.reshape(N, N0)
+    lhs, rhs = lhs.reshape(-1), rhs.reshape(-1)
+    init = np.zeros(M * N * M0 * N0, np.uint16)
+    flags = base | abi.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS
+    want = _oracle(oracle_lib, lhs, rhs, init, M, N, K, M0, N0, K0, flags)
+    d_l, d_r, d_o = (torch.from_numpy(x.view(np.int16)).cuda() for x in (lhs, rhs, init.copy()))
+    gpu_lib.iree_uk_mmt4d_p(C.byref(mm_params(d_l.data_ptr(), d_r.data_ptr(), d_o.data_ptr(), M, N, K, M0, N0, K0, flags)))
+    kernel = gpu_lib.iree_uk_mi355x_last_kernel()
+    assert b"generic" not in kernel
+    got = d_o.cpu().numpy().view(np.uint16)
+    # The cases the test is for are all present in what the reference produced.
+    emask = 0x7C00 if kind == "f16" else 0x7F80
+    field = want & emask
+    assert np.any((want & 0x7FFF) == 0) and np.any(field == emask)
+    if kind == "f16":   # (bf16 has f32's exponent range: below it there are only f32 subnormals, which give zero)
+        assert np.any((field == 0) & ((want & 0x7FFF) != 0))
+    assert len(np.unique(field)) >= (30 if kind == "f16" else 120)
+    bad = np.nonzero(got != want)[0]
+    assert bad.size == 0, (kernel, [(hex(int(got[i])), hex(int(want[i]))) for i in bad[:8]])
