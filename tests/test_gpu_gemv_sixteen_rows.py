@@ -60,3 +60,27 @@ def test_sixteen_row_lhs(gpu_lib, oracle_lib, case, acc):
         assert np.array_equal(got, want)
     else:
         assert_float_close(got, want, "16-row lhs N=%d K=%d K0=%d" % (N, K, K0))
+
+
+# Tile counts around the number of compute units (one workgroup per rhs tile: fewer workgroups than units, exactly
+# one or more per unit, the decode shape's 896), bit for bit on int8, with guard words either side of the output.
+@pytest.mark.parametrize("N", [256, 200, 128, 300, 896])
+@pytest.mark.parametrize("M0", [1, 4, 16])
+def test_tile_counts_around_the_number_of_compute_units(gpu_lib, oracle_lib, N, M0):
+    N0, K0, K = 16, 16, 24
+    flags = abi.MMT4D_TYPE_S8S8S32 | abi.MMT4D_ACCUMULATE
+    lhs = synth.uniform_int8(43, 0, K * M0 * K0)
+    rhs = synth.uniform_int8(43, 1, N * K * N0 * K0)
+    init = synth.uniform_int8(43, 2, N * M0 * N0).astype(np.int32) * 77
+    want = init.copy()
+    oracle_lib.oracle_mmt4d_mt(C.byref(mm_params(lhs.ctypes.data, rhs.ctypes.data, want.ctypes.data, 1, N, K, M0, N0, K0,
+                                                 flags | abi.MMT4D_ALLOW_GENERIC_FALLBACK)), 8)
+    d_l, d_r, d_o = torch.from_numpy(lhs).cuda(), torch.from_numpy(rhs).cuda(), torch.from_numpy(init.copy()).cuda()
+    guard = torch.full((64,), 123456, dtype=torch.int32, device="cuda")
+    d_all = torch.cat([guard, d_o, guard])
+    gpu_lib.iree_uk_mmt4d_p(C.byref(mm_params(d_l.data_ptr(), d_r.data_ptr(), d_all.data_ptr() + 256, 1, N, K, M0, N0, K0,
+                                              flags)))
+    assert gpu_lib.iree_uk_mi355x_last_kernel() == b"mmt4d_gemv"
+    got = d_all.cpu().numpy()
+    assert np.array_equal(got[64:-64], want)
+    assert (got[:64] == 123456).all() and (got[-64:] == 123456).all()
