@@ -41,6 +41,12 @@
 // (mmt4d_tile_generic.c:145-176): the rhs bytes are sign-extended to 16-bit
 // pairs (v_perm_b32 with its sign-byte selectors) for v_dot2_i32_i16.
 //
+// And s8s8s32 Mx8x1 with M0 = 1, 2, 4 (the Arm baseline tiles without dot
+// products, mmt4d_arm_64_tiles.inl:38-40): a k step of the rhs is 8 bytes, so a
+// lane's 16 bytes are the tile's 8 rows at two consecutive k steps; each row's
+// two bytes are put beside each other for one v_dot4_i32_i8 with the two lhs
+// bytes of those k steps.
+//
 // More than 8 lhs rows are worked off in slabs of 8, each streaming the rhs
 // again: what the block kernels can load they do faster (the caller prefers
 // them), what they cannot is still far better off here than with one thread
@@ -192,6 +198,13 @@ __device__ __forceinline__ void multiply_piece(const uint4 v, const typename Lhs
 #pragma unroll
       for (int i = 0; i < 2; ++i) acc[i] = dot2_i16(w[2 * i + 1], l.y, dot2_i16(w[2 * i], l.x, acc[i]));
     }
+  } else if constexpr (KIND == kI8 && G == 1) {
+    // 8 rows at k step 2j (bytes 0..7) and at 2j + 1 (bytes 8..15); l.x holds the two lhs bytes.
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const uint32_t pair = __builtin_amdgcn_perm(w[2 + (r >> 2)], w[r >> 2], 0x0C0C0400u + 0x0101u * (r & 3));
+      acc[r] = __builtin_amdgcn_sdot4((int)pair, (int)l.x, acc[r], false);
+    }
   } else if constexpr (KIND == kI8) {
     if constexpr (G == 2) {
       // Two rows per dword: the lhs pair in the low resp. high half, zeros in the other.
@@ -259,7 +272,9 @@ template <int KIND, int G, int ROWS, int UNROLL, bool NARROW>
 __global__ __launch_bounds__(256) void mmt4d_skinny_kernel(const SkinnyArgs a) {
   static_assert(!NARROW || KIND == kF16 || KIND == kBF16, "16-bit outputs are floats");
   typedef typename Acc<KIND>::type acc_t;
-  constexpr int R = 16 / G;  // rhs rows in a lane's 16 bytes
+  // (One-byte pieces of int8: 8-row tiles, two k steps per lane.)
+  constexpr bool TWO_KSTEPS = KIND == kI8 && G == 1;
+  constexpr int R = TWO_KSTEPS ? 8 : 16 / G;  // rhs rows in a lane's 16 bytes
   __shared__ acc_t partial[4][ROWS][32];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -267,8 +282,8 @@ __global__ __launch_bounds__(256) void mmt4d_skinny_kernel(const SkinnyArgs a) {
   // One k step of the rhs is N0 * G bytes = `lanes_per_kstep` lanes; a block of
   // 1 KiB holds whole k steps, so a lane keeps its rows from block to block.
   const int log2_kstep_bytes = a.log2_N0 + (G == 1 ? 0 : (G == 2 ? 1 : (G == 4 ? 2 : 3)));
-  const int log2_lanes_per_kstep = log2_kstep_bytes - 4;
-  const int32_t kstep_in_block = lane >> log2_lanes_per_kstep;
+  const int log2_lanes_per_kstep = TWO_KSTEPS ? 0 : log2_kstep_bytes - 4;
+  const int32_t kstep_in_block = TWO_KSTEPS ? 2 * lane : lane >> log2_lanes_per_kstep;
   constexpr int LHS_G = KIND == kI16U4 ? 16 : (KIND == kI8I4 || KIND == kI16I8 ? 2 * G : G);  // bytes of an lhs row piece
   const int32_t lhs_kstep_bytes = LHS_G << a.log2_M0;
 
@@ -295,12 +310,25 @@ __global__ __launch_bounds__(256) void mmt4d_skinny_kernel(const SkinnyArgs a) {
       const int64_t off = ((j0 + 4 * u) << 10) + 16 * lane;
       const bool inside = off < a.tile_bytes;
       v[u] = make_uint4(0, 0, 0, 0);
-      if (inside) v[u] = __builtin_bit_cast(uint4, __builtin_nontemporal_load((const v4i32*)(rhs_tile + off)));
+      if (TWO_KSTEPS && inside && off + 16 > a.tile_bytes) {
+        // An odd K: the stream ends after this lane's first k step.
+        const uint2 half = *(const uint2*)(rhs_tile + off);
+        v[u].x = half.x;
+        v[u].y = half.y;
+      } else if (inside) {
+        v[u] = __builtin_bit_cast(uint4, __builtin_nontemporal_load((const v4i32*)(rhs_tile + off)));
+      }
       // The lhs piece of this lane's k step.
       const int64_t kstep = inside ? ((j0 + 4 * u) << (10 - log2_kstep_bytes)) + kstep_in_block : 0;
 #pragma unroll
       for (int m = 0; m < ROWS; ++m) {
-        l[u][m] = load_lhs_piece<KIND, G>(lhs_row[m] + kstep * lhs_kstep_bytes);
+        if constexpr (TWO_KSTEPS) {
+          const uint8_t* p = lhs_row[m] + kstep * lhs_kstep_bytes;
+          const uint32_t second = kstep + 1 < a.K ? p[lhs_kstep_bytes] : 0u;
+          l[u][m] = make_uint2((uint32_t)p[0] | (second << 8), 0);
+        } else {
+          l[u][m] = load_lhs_piece<KIND, G>(lhs_row[m] + kstep * lhs_kstep_bytes);
+        }
         if (!inside) l[u][m] = typename LhsPiece<KIND>::type{};  // 0 * 0, whatever the lhs holds there
       }
     }
@@ -383,10 +411,13 @@ bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, int* piece_bytes,
   if (i4 && a.K0 != 2 && a.K0 != 8 && a.K0 != 16) return false;
   const int g = u4 ? 4 : (i4 ? a.K0 / 2 : (i16i8 ? a.K0 : a.K0 * elem_bytes));  // bytes of an rhs row piece
   const int lhs_g = u4 ? 16 : (i4 ? a.K0 : (i16i8 ? 2 * a.K0 : g));
-  if (g != 2 && g != 4 && g != 8 && !(i4 && g == 1)) return false;
+  // int8 Mx8x1 (8x8x1 goes to the matrix kernels first, see mmt4d_skinny_preferred, and comes here when they cannot
+  // load it: K shorter than a chunk, misaligned lhs).
+  const bool two_ksteps = *kind == kI8 && g == 1 && a.N0 == 8 && a.M0 <= 8;
+  if (g != 2 && g != 4 && g != 8 && !(i4 && g == 1) && !two_ksteps) return false;
   const int lm0 = log2_exact(a.M0), ln0 = log2_exact(a.N0);
-  // A k step of the rhs must be whole 16-byte vectors.
-  if (lm0 < 0 || ln0 < 0 || a.M0 > 16 || a.N0 > 32 || a.N0 * g < 16) return false;
+  // A k step of the rhs must be whole 16-byte vectors (or half of one, above).
+  if (lm0 < 0 || ln0 < 0 || a.M0 > 16 || a.N0 > 32 || (a.N0 * g < 16 && !two_ksteps)) return false;
   *piece_bytes = g;
   // What no matrix kernel takes.
   if (probe_only) return a.M0 * lhs_g < 16 || *kind == kI16 || u4 || i16i8 || (i4 && a.K0 < 16);
@@ -436,6 +467,9 @@ template <int KIND, bool NARROW>
 hipError_t launch_kind(const SkinnyArgs& s, int piece_bytes, hipStream_t stream) {
   if (piece_bytes == 4) return launch_piece<KIND, 4, NARROW>(s, stream);
   if (piece_bytes == 8) return launch_piece<KIND, 8, NARROW>(s, stream);
+  if constexpr (KIND == kI8) {
+    if (piece_bytes == 1) return launch_piece<KIND, 1, NARROW>(s, stream);
+  }
   if constexpr (KIND != kF32) return launch_piece<KIND, 2, NARROW>(s, stream);
   return hipErrorInvalidValue;
 }
@@ -471,7 +505,9 @@ hipError_t launch_skinny(const Mmt4dArgs& a, hipStream_t stream, const char** na
 bool mmt4d_skinny_preferred(const Mmt4dArgs& a) {
   int lhs_bits, rhs_bits, out_bits;
   if (!mmt4d_type_bits(a.flags, &lhs_bits, &rhs_bits, &out_bits)) return false;
-  return a.M * a.M0 <= 4 || a.M0 * a.K0 * lhs_bits / 8 < 16;
+  // (8-row tiles of one-byte pieces are 8 bytes per k step, but the matrix kernels load them k-major.)
+  const bool k_major_for_mfma = a.K0 * lhs_bits == 8 && a.M0 >= 8;
+  return a.M * a.M0 <= 4 || (a.M0 * a.K0 * lhs_bits / 8 < 16 && !k_major_for_mfma);
 }
 
 Mmt4dLauncher select_mmt4d_skinny(const Mmt4dArgs& a, bool probe_only) {

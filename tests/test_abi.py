@@ -211,13 +211,13 @@ def test_mmt4d_info_reports_specialised_kernels():
                             (abi.MMT4D_TYPE_S16S16S32, 1, 16, 2), (abi.MMT4D_TYPE_S16S16S32, 16, 16, 2), (abi.MMT4D_TYPE_S16U4S32, 1, 32, 8),
                             (abi.MMT4D_TYPE_S8S4S32, 4, 8, 8), (abi.MMT4D_TYPE_S8S4S32, 1, 8, 16),
                             (abi.MMT4D_TYPE_S8S4S32, 4, 16, 2), (abi.MMT4D_TYPE_S16S8S32, 16, 16, 2),
-                            (abi.MMT4D_TYPE_S16S8S32, 1, 8, 8)]:
+                            (abi.MMT4D_TYPE_S16S8S32, 1, 8, 8), (abi.MMT4D_TYPE_S8S8S32, 4, 8, 1)]:
         assert lib.iree_uk_mmt4d_info(m0, n0, k0, t, None) == 1, (hex(t), m0, n0, k0)
     assert lib.iree_uk_mmt4d_info(9, 6, 3, abi.MMT4D_TYPE_S8S8S32, None) == 0
     assert lib.iree_uk_mmt4d_info(8, 8, 4, 0x0B, None) == 0
-    # What only the generic kernel takes: one-byte row pieces in tiles less than 8 rows tall, tile sizes that are
-    # not powers of two (the reference tests s16s8s32 on 7x5x6), f16f16f16 with a rounding after every k step.
-    assert lib.iree_uk_mmt4d_info(4, 8, 1, abi.MMT4D_TYPE_S8S8S32, None) == 0
+    # What only the generic kernel takes: tile sizes that are not powers of two (the reference tests s16s8s32 on
+    # 7x5x6), one-byte row pieces in shapes no CPU target uses, f16f16f16 with a rounding after every k step.
+    assert lib.iree_uk_mmt4d_info(4, 4, 1, abi.MMT4D_TYPE_S8S8S32, None) == 0
     assert lib.iree_uk_mmt4d_info(8, 8, 1, abi.MMT4D_TYPE_S8S8S32, None) == 1   # k-major int8: transposing LDS reads
     assert lib.iree_uk_mmt4d_info(7, 5, 6, abi.MMT4D_TYPE_S16S8S32, None) == 0
     assert lib.iree_uk_mmt4d_info(16, 16, 1, abi.MMT4D_TYPE_F16F16F16, None) == 0
@@ -234,3 +234,23 @@ def test_query_tile_sizes_roles_are_consistent():
         n0, k0r = query(op | abi.QTS_ROLE_RHS)
         assert k0 == k0r
         assert query(op | abi.QTS_ROLE_RESULT) == (m0, n0)
+
+
+def test_every_tile_shape_of_the_reference_cpu_targets_has_a_specialised_kernel():
+    # tests/golden/reference_arch_tiles.json lists the reference's tables of architecture-specific tile functions
+    # (mmt4d_x86_64_tiles.inl, mmt4d_arm_64_tiles.inl; written by tests/golden/make_tile_list.py): the tile shapes a
+    # caller compiled for those CPUs passes. None of them may end up on the one-thread-per-element kernel.
+    import json
+    import os
+    lib = library.load()
+    skip = abi.MMT4D_SKIP_INTERMEDIATE_ROUNDINGS   # what the compiler sets for 16-bit outputs
+    flag = {"f32f32f32": abi.MMT4D_TYPE_F32F32F32, "f16f16f32": abi.MMT4D_TYPE_F16F16F32,
+            "f16f16f16": abi.MMT4D_TYPE_F16F16F16 | skip, "bf16bf16f32": abi.MMT4D_TYPE_BF16BF16F32,
+            "bf16bf16bf16": abi.MMT4D_TYPE_BF16BF16BF16 | skip, "s8s8s32": abi.MMT4D_TYPE_S8S8S32,
+            "s16s16s32": abi.MMT4D_TYPE_S16S16S32, "s16u4s32": abi.MMT4D_TYPE_S16U4S32, "s8s4s32": abi.MMT4D_TYPE_S8S4S32}
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_arch_tiles.json")
+    tiles = json.load(open(path))["tiles"]
+    assert len(tiles) >= 90 and {t["arch"] for t in tiles} == {"x86_64", "arm_64"}
+    missing = [(t["arch"], t["type"], t["M0"], t["N0"], t["K0"]) for t in tiles
+               if lib.iree_uk_mmt4d_info(t["M0"], t["N0"], t["K0"], flag[t["type"]], None) != 1]
+    assert not missing, missing

@@ -57,8 +57,9 @@ def test_odd_k_with_16_row_tiles(gpu_lib):
 
 
 def test_what_the_transposing_path_does_not_take_stays_exact(gpu_lib):
-    # less than one chunk of K, 4-row tiles, operands that are not 16-byte aligned: the generic kernel
-    run_case(gpu_lib, S8, 5, 4, 40, 8, 8, 1, "mmt4d_generic", accumulate=True)
-    run_case(gpu_lib, S8, 5, 4, 100, 4, 8, 1, "mmt4d_generic")
-    run_case(gpu_lib, S8, 5, 4, 100, 8, 8, 1, "mmt4d_generic", offsets=(8, 0, 0))
+    # less than one chunk of K, 4-row tiles, an lhs that is not 16-byte aligned: the narrow-tile kernel
+    # (tests/test_gpu_skinny_narrow.py); rhs tile rows that are not 16-byte multiples apart: the generic kernel
+    run_case(gpu_lib, S8, 5, 4, 40, 8, 8, 1, "mmt4d_skinny", accumulate=True)
+    run_case(gpu_lib, S8, 5, 4, 100, 4, 8, 1, "mmt4d_skinny")
+    run_case(gpu_lib, S8, 5, 4, 100, 8, 8, 1, "mmt4d_skinny", offsets=(8, 0, 0))
     run_case(gpu_lib, S8, 5, 4, 129, 8, 8, 1, "mmt4d_generic")

@@ -156,6 +156,21 @@ def test_int4_weights_in_narrow_tiles(gpu_lib, M, M0, N0, K0):
              accumulate=True, seed=3)
 
 
+# int8 Mx8x1, the Arm tiles without dot products (mmt4d_arm_64_tiles.inl:38-40): a k step of the rhs is 8 bytes, two
+# per lane. Even K, odd K (the stream ends inside a lane's 16 bytes; rhs tile rows padded to 16-byte multiples), more
+# rows than one slab, strides and offsets, accumulate.
+@pytest.mark.parametrize("M,M0", [(1, 1), (1, 2), (1, 4), (3, 1), (5, 4)])
+def test_int8_one_byte_pieces_in_tiles_of_up_to_four_rows(gpu_lib, M, M0):
+    for n, K in enumerate((2, 64, 130, 2000)):
+        run_case(gpu_lib, S8, M, 33 + n, K, M0, 8, 1, "mmt4d_skinny", accumulate=bool(n & 1), seed=K + M0)
+    for n, K in enumerate((1, 77, 1501)):
+        run_case(gpu_lib, S8, M, 21 + n, K, M0, 8, 1, "mmt4d_skinny", rhs_pad=8, accumulate=not (n & 1), seed=K)
+    run_case(gpu_lib, S8, M, 19, 131, M0, 8, 1, "mmt4d_skinny", lhs_pad=3, rhs_pad=24, out_pad=5, offsets=(5, 48, 3),
+             accumulate=True, seed=11)
+    # rhs tile rows that are not 16-byte multiples apart: the generic kernel
+    run_case(gpu_lib, S8, M, 7, 77, M0, 8, 1, "mmt4d_generic")
+
+
 def test_sixteen_bit_integer_types_with_more_rows_are_worked_off_in_slabs(gpu_lib):
     # No matrix kernel exists for them: any number of rows goes through this kernel eight rows at a time, also the
     # 16-row tiles of the x86-64 VNNI target (s16s16s32 16x16x2, mmt4d_x86_64_tiles.inl:69,74).
