@@ -912,10 +912,50 @@ hipError_t launch_pack(const PackArgs& original, hipStream_t stream, const char*
     a.out_size2 = 1;
     tr_inner = false;
   }
+  // Tiles of 8 bytes with a unit dimension (int8 8x1, the Arm tiles for K0 = 1,
+  // arch/arm_64/pack_arm_64_entry_point.c:24-26): the vectors of the tiled side
+  // are 16 bytes, i.e. two tiles that follow each other along out dimension 1,
+  // and two such tiles are one 16-byte tile: [1][n] twice along the direction
+  // of n is [1][2n]; along the other direction it is [2][n]. With an odd
+  // number of tiles along that dimension the last one is left to the generic
+  // kernel (a slice of the source and one column of tiles).
+  PackArgs last_tiles;
+  bool have_last_tiles = false;
+  if (a.out_size2 * a.out_size3 * a.elem_bytes == 8 && (a.out_size2 == 1 || a.out_size3 == 1) &&
+      a.out_size1 >= 2 && a.in_stride1 == 1) {
+    if (a.out_size3 == 1) {  // [n][1] is [1][n] with the other inner order
+      a.out_size3 = a.out_size2;
+      a.out_size2 = 1;
+      tr_inner = !tr_inner;
+    }
+    const int merge_dim = tr_outer ? 0 : 1;   // source dimension that out dimension 1 walks along
+    const int long_dim = tr_inner ? 0 : 1;    // source dimension of the tile's n elements
+    const int64_t tile_extent = merge_dim == long_dim ? a.out_size3 : 1;
+    if (a.out_size1 & 1) {
+      const int64_t start = (a.out_size1 - 1) * tile_extent;  // first source coordinate of the last tiles
+      int64_t& size_along = merge_dim == 0 ? a.in_size0 : a.in_size1;
+      last_tiles = a;
+      last_tiles.flags = (a.flags & ~(uint32_t)IREE_UK_FLAG_PACK_TRANSPOSE_INNER) |
+                         (tr_inner ? IREE_UK_FLAG_PACK_TRANSPOSE_INNER : 0u);
+      last_tiles.in = a.in + start * (merge_dim == 0 ? a.in_stride0 : a.in_stride1) * a.elem_bytes;
+      (merge_dim == 0 ? last_tiles.in_size0 : last_tiles.in_size1) = size_along > start ? size_along - start : 0;
+      last_tiles.out = a.out + (a.out_size1 - 1) * 8;
+      last_tiles.out_size1 = 1;
+      have_last_tiles = true;
+      size_along = size_along < start ? size_along : start;
+      a.out_size1 -= 1;
+    }
+    a.out_size1 /= 2;
+    if (merge_dim == long_dim) a.out_size3 *= 2; else a.out_size2 = 2;
+  }
   if (!make_plan(a.in, a.out, a.in_stride0, a.in_stride1, a.out_stride0, a.in_size0, a.in_size1,
                  a.out_size0, a.out_size1, a.out_size2, a.out_size3, tr_inner, tr_outer,
                  a.elem_bytes, /*for_unpack=*/false, &plan))
     return launch_pack_generic(original, stream, name);
+  if (have_last_tiles) {
+    const hipError_t e = launch_pack_generic(last_tiles, stream, name);
+    if (e != hipSuccess) return e;
+  }
   plan.args.src = a.in;
   plan.args.dst = a.out;
   plan.args.padding_value = a.padding_value;

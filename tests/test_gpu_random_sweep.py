@@ -200,3 +200,100 @@ def test_mmt4d_random_cases_more_types_and_shapes(gpu_lib, oracle_lib):
              abi.MMT4D_TYPE_F32F32F32, abi.MMT4D_TYPE_F16F16F16 | skip, abi.MMT4D_TYPE_BF16BF16BF16 | skip]
     kernels = _mmt4d_sweep(gpu_lib, oracle_lib, 21, 300, types, [2, 4, 8, 16, 16], long_k=True)
     assert {b"mmt4d_generic", b"mmt4d_mfma_64x64", b"mmt4d_skinny"} <= kernels
+
+
+# The tile shapes for which the reference's x86-64 and Arm targets have their own pack / unpack tile functions
+# (arch/x86_64/pack_x86_64_entry_point.c:99-113, arch/arm_64/pack_arm_64_entry_point.c:16-31; unpack:
+# arch/x86_64/unpack_x86_64_entry_point.c:18-30, arch/arm_64/unpack_arm_64_entry_point.c:13-19), as (element bytes,
+# out_size2, out_size3): what a caller compiled for those CPUs passes. Each with every transpose combination, on a
+# ragged matrix, bit for bit against the oracle, and none of them on a one-thread-per-element kernel.
+CPU_PACK_TILES = [(4, 8, 8), (4, 16, 16), (4, 8, 1), (4, 16, 1), (2, 16, 2), (1, 8, 2), (1, 16, 2), (1, 8, 1), (1, 8, 4),
+                  (1, 8, 8)]
+CPU_UNPACK_TILES = [(4, 8, 8), (4, 16, 16)]
+
+
+@pytest.mark.parametrize("e,s2,s3", CPU_PACK_TILES)
+@pytest.mark.parametrize("flags", [0, TI, TO, TI | TO])
+def test_pack_tile_shapes_of_the_reference_cpu_targets(gpu_lib, oracle_lib, e, s2, s3, flags):
+    typ = {4: abi.PACK_TYPE_F32F32, 2: abi.PACK_TYPE_BF16BF16, 1: abi.PACK_TYPE_I8I8}[e]
+    t0, t1 = (s3, s2) if flags & TI else (s2, s3)      # tile extents along dims 0 and 1 of the source
+    rows, cols = 1276, 2044     # (8-byte tiles are taken in pairs: an even number of them whichever way they run)
+    o0, o1 = -(-rows // t0), -(-cols // t1)
+    s0, s1 = (o1, o0) if flags & TO else (o0, o1)
+    out_stride = s1 * s2 * s3
+    src = np.frombuffer(np.random.default_rng(e * 100 + s2 + s3 + flags).bytes(rows * cols * e), dtype=np.int8).copy()
+
+    def pack_params(src_ptr, dst_ptr):
+        p = abi.PackParams()
+        p.in_buffer, p.out_buffer = src_ptr, dst_ptr
+        p.in_stride0, p.in_stride1 = cols, 1
+        p.out_stride0, p.out_stride1 = out_stride, s2 * s3
+        p.in_size0, p.in_size1 = rows, cols
+        p.out_size0, p.out_size1, p.out_size2, p.out_size3 = s0, s1, s2, s3
+        p.padding_value = 0x5AA55AA5
+        p.flags = typ | flags
+        return p
+
+    want = np.full(s0 * out_stride * e, 0x77, dtype=np.int8)
+    oracle_lib.oracle_pack(C.byref(pack_params(src.ctypes.data, want.ctypes.data)))
+    d_src = torch.from_numpy(src).cuda()
+    d_out = torch.full((want.size,), 0x77, dtype=torch.int8, device="cuda")
+    gpu_lib.iree_uk_pack_p(C.byref(pack_params(d_src.data_ptr(), d_out.data_ptr())))
+    kernel = gpu_lib.iree_uk_mi355x_last_kernel()
+    assert np.array_equal(d_out.cpu().numpy(), want)
+    assert kernel and b"generic" not in kernel, kernel
+    if (e, s2, s3) not in CPU_UNPACK_TILES or flags:
+        return
+    back = np.full(rows * cols * e, 0x33, dtype=np.int8)
+
+    def unpack_params(src_ptr, dst_ptr):
+        p = abi.UnpackParams()
+        p.in_buffer, p.out_buffer = src_ptr, dst_ptr
+        p.in_stride0, p.in_stride1 = out_stride, s2 * s3
+        p.out_stride0, p.out_stride1 = cols, 1
+        p.in_size0, p.in_size1, p.in_size2, p.in_size3 = s0, s1, s2, s3
+        p.out_size0, p.out_size1 = rows, cols
+        p.flags = abi.UNPACK_TYPE_F32F32
+        return p
+
+    d_back = torch.full((back.size,), 0x33, dtype=torch.int8, device="cuda")
+    gpu_lib.iree_uk_unpack_p(C.byref(unpack_params(d_out.data_ptr(), d_back.data_ptr())))
+    kernel = gpu_lib.iree_uk_mi355x_last_kernel()
+    assert np.array_equal(d_back.cpu().numpy(), src)
+    assert kernel and b"generic" not in kernel, kernel
+
+
+@pytest.mark.parametrize("flags", [0, TI, TO, TI | TO])
+def test_eight_byte_tiles_with_an_odd_tile_count(gpu_lib, oracle_lib, flags):
+    # int8 8x1 tiles are taken two at a time; with an odd number of them along out dimension 1 the last column of
+    # tiles is written by a second launch. Rows of the tiled buffer padded to 16-byte multiples; the whole
+    # destination (pre-filled) is compared, padding tiles beyond the source included.
+    s2, s3 = 8, 1
+    t0, t1 = (s3, s2) if flags & TI else (s2, s3)
+    rows, cols = 1237, 2041
+    o0, o1 = -(-rows // t0) + 2, -(-cols // t1)       # two rows of tiles that are nothing but padding
+    if ((o0 if flags & TO else o1) & 1) == 0:
+        o0, o1 = (o0 + 1, o1) if flags & TO else (o0, o1 + 1)
+    s0, s1 = (o1, o0) if flags & TO else (o0, o1)
+    assert s1 & 1
+    out_stride = s1 * 8 + 8
+    src = np.frombuffer(np.random.default_rng(flags + 5).bytes(rows * cols), dtype=np.int8).copy()
+
+    def pack_params(src_ptr, dst_ptr):
+        p = abi.PackParams()
+        p.in_buffer, p.out_buffer = src_ptr, dst_ptr
+        p.in_stride0, p.in_stride1 = cols, 1
+        p.out_stride0, p.out_stride1 = out_stride, 8
+        p.in_size0, p.in_size1 = rows, cols
+        p.out_size0, p.out_size1, p.out_size2, p.out_size3 = s0, s1, s2, s3
+        p.padding_value = 0x5A
+        p.flags = abi.PACK_TYPE_I8I8 | flags
+        return p
+
+    want = np.full(s0 * out_stride, 0x77, dtype=np.int8)
+    oracle_lib.oracle_pack(C.byref(pack_params(src.ctypes.data, want.ctypes.data)))
+    d_src = torch.from_numpy(src).cuda()
+    d_out = torch.full((want.size,), 0x77, dtype=torch.int8, device="cuda")
+    gpu_lib.iree_uk_pack_p(C.byref(pack_params(d_src.data_ptr(), d_out.data_ptr())))
+    assert gpu_lib.iree_uk_mi355x_last_kernel() in (b"pack_tiled", b"pack_transposing")
+    assert np.array_equal(d_out.cpu().numpy(), want)
