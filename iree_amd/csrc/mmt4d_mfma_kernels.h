@@ -694,13 +694,28 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
     const int64_t tile = (row >> log2_t0) - (first >> log2_t0);
     return tile * stride_bytes + (row & ((1 << log2_t0) - 1)) * rb;
   };
+  //   G == 16, lhs tiles one row tall (a row-major matrix: a row's 64 bytes of a
+  //     chunk are contiguous, consecutive rows a whole row pitch apart): with the
+  //     arrangement above four consecutive lanes would load from four cache
+  //     lines. Here lane l of a load takes row l >> 2 of the load's 16 and the
+  //     16-byte column (l & 3) ^ ((l >> 4) & 3), so four consecutive lanes cover
+  //     one row's 64 bytes; lane 32*h + r reads slot 128*f + 64*(r >> 4) + 4*r' +
+  //     ((2*kk + h) ^ ((r' >> 2) & 3)), r' = r & 15: the xor spreads the sixteen
+  //     rows of a group of lanes over all banks. The slot for K-step 1 is the one
+  //     for K-step 0 with bit 1 flipped, a per-lane distance (lhs_kk1_step).
+  constexpr bool ROWS16 = G == 16 && !RHS_I4;
+  const bool lhs_row_major = ROWS16 && a.log2_M0 == 0;
   uint32_t a_off[A_LOADS], b_off[B_LOADS];
   if constexpr (G == 16) {
 #pragma unroll
     for (int t = 0; t < A_LOADS; ++t) {
       const int p = tid + 256 * t;
-      const int c = RHS_I4 ? ((p >> 6) & 1) + 2 * ((p >> 5) & 1) : (p >> 4) & 3;
-      const int row = RHS_I4 ? (p >> 7) * 32 + (p & 31) : (p >> 7) * 32 + 16 * ((p >> 6) & 1) + (p & 15);
+      int c = RHS_I4 ? ((p >> 6) & 1) + 2 * ((p >> 5) & 1) : (p >> 4) & 3;
+      int row = RHS_I4 ? (p >> 7) * 32 + (p & 31) : (p >> 7) * 32 + 16 * ((p >> 6) & 1) + (p & 15);
+      if (lhs_row_major) {
+        c = (p & 3) ^ ((p >> 4) & 3);
+        row = (p >> 7) * 32 + 16 * ((p >> 6) & 1) + ((p >> 2) & 15);
+      }
       a_off[t] = (uint32_t)(row_offset(first_row + row, total_rows - 1, first_row,
                                        a.log2_M0, a.lhs_stride_bytes, a.lhs_rb) +
                             ((16 * c) >> a.log2_lhs_rb) * lhs_kstep + ((16 * c) & (a.lhs_rb - 1)));
@@ -840,6 +855,8 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
       return widen_i4_times16(kk ? make_uint2(raw.z, raw.w) : make_uint2(raw.x, raw.y));
     }
     if constexpr (G == 16) {
+      if (!RHS_I4 && operand == 0 && lhs_row_major)
+        return ring[128 * f + 64 * ((lane & 31) >> 4) + 4 * (lane & 15) + ((2 * kk + (lane >> 5)) ^ ((lane >> 2) & 3))];
       if (!RHS_I4) return ring[operand + 128 * f + 32 * kk + 64 * ((lane & 31) >> 4) + 16 * (lane >> 5) + (lane & 15)];
       return ring[operand + 128 * f + 64 * kk + lane];
     } else if constexpr (G == 1) {
@@ -881,7 +898,6 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   const uint32_t frag_b_off = (uint32_t)(A_PIECES + (wave_n * BN) * (RHS_I4 ? 64 : 128)) * 16;
   // Lane 32*h + r's byte offset into a fragment, and the slots from one K-step
   // of a fragment to the next (see the layouts above).
-  constexpr bool ROWS16 = G == 16 && !RHS_I4;
   const uint8_t* ring_bytes =
       (const uint8_t*)ring + (ROWS16 ? 16 * (64 * ((lane & 31) >> 4) + 16 * (lane >> 5) + (lane & 15))
                                      : (G == 1 ? 0 : (G == 16 ? 16 : G) * lane));
@@ -892,8 +908,14 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   // tiles 1.8x slower than the 4-byte ones: the second read of a register has
   // to wait for the first.)
   // (G == 1: the per-operand lane offset of the transposing reads instead.)
+  // (Row-major lhs: the distance from the rhs lane slot, which ring_bytes holds, to the lhs one for K-step 0.)
+  const int32_t lhs_rm_slot0 = 4 * (lane & 15) + ((lane >> 5) ^ ((lane >> 2) & 3));
   const int32_t pair_a_lane =
-      G == 1 ? transposed_lane_offset(a.log2_M0) : (G != 2 ? 0 : (PAIR_A ? 2 * lane : -2 * (lane & 1)));
+      G == 1 ? transposed_lane_offset(a.log2_M0)
+             : (G == 2 ? (PAIR_A ? 2 * lane : -2 * (lane & 1))
+                       : (lhs_row_major ? 16 * (lhs_rm_slot0 - (16 * (lane >> 5) + (lane & 15))) : 0));
+  // Bytes from an lhs fragment's K-step 0 to its K-step 1 in this lane's reads.
+  const int32_t lhs_kk1_step = lhs_row_major ? 16 * ((lhs_rm_slot0 ^ 2) - lhs_rm_slot0) : 16 * (ROWS16 ? 32 : 64);
   const int32_t pair_b_lane =
       G == 1 ? transposed_lane_offset(a.log2_N0) : (G != 2 ? 0 : (PAIR_B ? 2 * lane : -2 * (lane & 1)));
   const uint32_t own_half = (lane & 1) ? 0x07060302u : 0x05040100u;
@@ -975,6 +997,7 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
     // The fragments read during this step are those of chunk load_chunk - AHEAD + 1.
     const bool cut_next = cut_bytes != 0 && load_chunk - AHEAD + 1 == last_chunk;
     const uint8_t* read_a = ring_bytes + read_stage_off + frag_a_off + pair_a_lane;
+    const uint8_t* read_a_kk1 = read_a + lhs_kk1_step;  // (used where the lhs has 16-byte pieces)
     const uint8_t* read_b = ring_bytes + read_stage_off + frag_b_off + pair_b_lane;
     uint4 raw_b[RHS_I4 ? BN : 1];
 #pragma unroll
@@ -992,7 +1015,7 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
               raw_b[u] = *(const uint4*)(read_b + (64 * u) * 16);
             } else {
               const int kk = (u - B_UNITS) / AM, i = (u - B_UNITS) % AM;
-              nxt_a[i][kk] = *(const uint4*)(read_a + (128 * i + KK16 * kk) * 16);
+              nxt_a[i][kk] = *(const uint4*)((kk ? read_a_kk1 : read_a) + 128 * i * 16);
             }
           } else {
             bool is_b, paired;
@@ -1007,7 +1030,8 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
             const int frag = y / PARTS, part = y % PARTS;
             uint4& dst = nxt[frag][kk];
             if constexpr (G == 16) {
-              dst = *(const uint4*)(src + (128 * frag + KK16 * kk) * 16);
+              if (is_b) dst = *(const uint4*)(src + (128 * frag + KK16 * kk) * 16);
+              else dst = *(const uint4*)((kk ? read_a_kk1 : read_a) + 128 * frag * 16);
             } else {
               const uint8_t* first = src + 1024 * (2 * frag + kk);
               if constexpr (G == 1) {

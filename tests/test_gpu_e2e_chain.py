@@ -125,3 +125,66 @@ def test_pack_mmt4d_unpack_equals_row_major_matmul(gpu_lib, kind, M, N, K, accum
     else:
         assert torch.equal(c[:M, :N].double(), want), kernels
     assert bool((c[M, :] == 55).all()) and bool((c[:, N] == 55).all())
+
+
+@pytest.mark.parametrize("kind", ["i8", "f16", "bf16", "f32"])
+@pytest.mark.parametrize("M,N,K", [(301, 517, 1000), (1, 4097, 130), (600, 33, 77), (1025, 1023, 2050), (256, 512, 4096)])
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_row_major_lhs_and_result_need_no_pack_or_unpack(gpu_lib, kind, M, N, K, accumulate):
+    """The fused form of the chain: a row-major [M, K] matrix IS the mmt4d lhs [M][K1][1][K0] (tiles one row
+    tall follow each other along the row), and the mmt4d result [M][N1][1][N0] IS the row-major [M, N1*N0]
+    matrix, so with M0 = 1 only the rhs is packed (mmt4d.c:12-48 puts no lower bound on M0; operand
+    addressing mmt4d.c:55-99). Same comparison as above, tools/e2e_matmul_benchmark.c:340-358. K is padded
+    to whole tiles by the row pitch of the lhs; what lies in that padding meets the zero padding of the
+    packed rhs."""
+    op, mm_type, in_pack, _, _, in_dtype, out_dtype = KINDS[kind]
+    (_, k0), (n0, _) = (_query(gpu_lib, op, r) for r in (abi.QTS_ROLE_LHS, abi.QTS_ROLE_RHS))
+    N1, K1 = -(-N // n0), -(-K // k0)
+    g = torch.Generator(device="cuda").manual_seed(M * 7 + N * 3 + K + (1 if accumulate else 0))
+    if kind == "i8":
+        a = torch.randint(-128, 128, (M, K), dtype=torch.int8, device="cuda", generator=g)
+        b = torch.randint(-128, 128, (K, N), dtype=torch.int8, device="cuda", generator=g)
+        init = torch.randint(-100000, 100000, (M, N), dtype=torch.int32, device="cuda", generator=g)
+    else:
+        a = torch.randint(-3, 4, (M, K), device="cuda", generator=g).to(in_dtype)
+        b = torch.randint(-3, 4, (K, N), device="cuda", generator=g).to(in_dtype)
+        init = torch.randint(-1000, 1000, (M, N), device="cuda", generator=g).to(out_dtype)
+    # lhs rows padded to whole tiles with something that is not zero; one guard row after the matrix.
+    a_pitch = K1 * k0
+    a_rm = torch.full((M + 1, a_pitch), 7, dtype=in_dtype, device="cuda")
+    a_rm[:M, :K] = a
+    b4 = torch.full((N1 * K1 * n0 * k0,), 7, dtype=in_dtype, device="cuda")
+    # Result: rows of N1*N0 values, pitch with 5 guard columns, one guard row.
+    c_pitch = N1 * n0 + 8
+    c = torch.full((M + 1, c_pitch), 55, dtype=out_dtype, device="cuda")
+    if accumulate:
+        c[:M, :N] = init
+        c[:M, N:N1 * n0] = 0
+    kernels = []
+
+    def call(fn, p):
+        fn(C.byref(p))
+        kernels.append(gpu_lib.iree_uk_mi355x_last_kernel().decode())
+
+    call(gpu_lib.iree_uk_pack_p, _pack(b, b4, K, N, N1, K1, n0, k0,
+                                       in_pack | abi.PACK_TRANSPOSE_INNER | abi.PACK_TRANSPOSE_OUTER))
+    p = abi.Mmt4dParams()
+    p.lhs_buffer, p.rhs_buffer, p.out_buffer = a_rm.data_ptr(), b4.data_ptr(), c.data_ptr()
+    p.lhs_stride0, p.rhs_stride0, p.out_stride0 = a_pitch, K1 * n0 * k0, c_pitch
+    p.M, p.N, p.K, p.M0, p.N0, p.K0 = M, N1, K1, 1, n0, k0
+    p.flags = mm_type | (abi.MMT4D_ACCUMULATE if accumulate else 0)
+    call(gpu_lib.iree_uk_mmt4d_p, p)
+    assert all(k and "generic" not in k for k in kernels), kernels
+    assert kernels[1].startswith("mmt4d_mfma") or kernels[1].startswith("mmt4d_gemv") or \
+        kernels[1].startswith("mmt4d_skinny"), kernels
+
+    want = a.double() @ b.double()
+    if accumulate:
+        want = want + init.double()
+    if kind == "i8":
+        want = ((want.long() + 2 ** 31) % 2 ** 32 - 2 ** 31)
+        assert torch.equal(c[:M, :N].long(), want), kernels
+    else:
+        assert torch.equal(c[:M, :N].double(), want), kernels
+    assert bool((c[:M, N:N1 * n0] == 0).all()), "columns of the padded rhs rows are zero"
+    assert bool((c[M, :] == 55).all()) and bool((c[:, N1 * n0:] == 55).all())
