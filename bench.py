@@ -165,9 +165,29 @@ def _e2e_chain(torch, lib, abi, synth, steps, warmup):
     rows = [0, 1777, 4095]
     ref_rows = (a.view(S, S)[rows].double() @ b.view(S, S).double()).long()
     ok = bool(c.to(torch.int64).sum().item() == want) and bool(torch.equal(c.view(S, S)[rows].long(), ref_rows))
+
+    # The fused form: a row-major [M, K] matrix is the mmt4d lhs [M][K1][1][K0] as it stands, and the
+    # result [M][N1][1][N0] is the row-major [M, N] matrix, so with tiles one row tall only the rhs
+    # is packed: two launches instead of four, no packed copy of the lhs or of the result.
+    c_fused = torch.empty(S * S, dtype=torch.int32, device="cuda")
+    p_rm = _mmt4d_params(abi, a.data_ptr(), b4.data_ptr(), c_fused.data_ptr(), S, N1, K1, 1, n0, k0,
+                         abi.MMT4D_TYPE_S8S8S32)
+    timed("mmt4d_row_major_lhs_and_result", lambda: lib.iree_uk_mmt4d_p(C.byref(p_rm)))
+
+    def fused():
+        lib.iree_uk_pack_p(C.byref(p_rhs))
+        lib.iree_uk_mmt4d_p(C.byref(p_rm))
+    fused_ms, _ = _time_launches(torch, fused, steps, warmup)
+    fused_ok = bool(torch.equal(c_fused, c))
     return {"tiles": "%dx%dx%d" % (m0, n0, k0), "ms": round(ms, 5), "value": round(2.0 * S ** 3 / ms / 1e9, 1),
             "unit": "TOP/s", "frac_of_peak": round(2.0 * S ** 3 / ms / 1e9 / PEAK_INT8_TOPS, 4),
-            "equals_row_major_product": ok, "parts": parts}
+            "equals_row_major_product": ok, "parts": parts,
+            "fused_row_major_lhs_and_result": {
+                "what": "pack rhs, then mmt4d with tiles 1x%dx%d reading the row-major lhs and writing the "
+                        "row-major result (no pack of the lhs, no unpack)" % (n0, k0),
+                "ms": round(fused_ms, 5), "value": round(2.0 * S ** 3 / fused_ms / 1e9, 1), "unit": "TOP/s",
+                "frac_of_peak": round(2.0 * S ** 3 / fused_ms / 1e9 / PEAK_INT8_TOPS, 4),
+                "equals_unfused_result": fused_ok}}
 
 
 def _also(torch, lib, abi, synth, steps, warmup):

@@ -70,10 +70,12 @@ typedef long long iree_uk_index_t;
 #define IREE_UK_FLAG_UNPACK_TRANSPOSE_OUTER 0x200
 
 #define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_MASK 0xFF
+#define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_NONE 0x00
 #define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_LHS 0x01
 #define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_RHS 0x02
 #define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERAND_ROLE_RESULT 0x03
 #define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MASK 0xFF00
+#define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERATION_NONE 0x0000
 #define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_F32F32F32 0x0100
 #define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_I8I8I32 0x0200
 #define IREE_UK_FLAG_QUERY_TILE_SIZES_OPERATION_MATMUL_F16F16F32 0x0300
@@ -251,9 +253,9 @@ int iree_uk_mi355x_multi_mma_i32_16x16x64_i8(const void* a, const void* b, void*
 
 /* iree_uk_mmt4d_p for callers that cannot allocate. It has no counterpart in
  * the reference (whose microkernels never allocate, being CPU code); it is for
- * callers that may not call hipMalloc where they call a microkernel: code
- * under HIP graph capture, tight serving loops, harnesses that forbid
- * allocation. Same parameters, checks, kernels and results as iree_uk_mmt4d_p.
+ * callers that may not call hipMalloc where they call a microkernel: tight
+ * serving loops, harnesses that forbid allocation, code around HIP graph
+ * capture. Same parameters, checks, kernels and results as iree_uk_mmt4d_p.
  * The difference: operands at host addresses are mirrored in a fixed array of
  * IREE_UK_MI355X_NOALLOC_MAX_STAGED_BYTES of device memory that the library's
  * code object holds on every device it runs on until the process ends, instead
@@ -262,10 +264,19 @@ int iree_uk_mi355x_multi_mma_i32_16x16x64_i8(const void* a, const void* b, void*
  * operands need more in total reports "host operands exceed ..." through the
  * failure handler and returns without launching. Device operands take none.
  * The call makes no hipMalloc/hipFree. All calls on one device share that
- * array: calls that overlap in time on one device race (serialise them); the
- * array keeps the previous call's bytes, and nothing read from it is ever
- * older than the current call's own uploads. iree_uk_mi355x_init resolves
- * the array's address ahead of the first call. */
+ * array, one at a time: a call with host operands holds it from its first
+ * upload until its results are back on the host, and a second such call that
+ * arrives on the same device meanwhile (from another thread) is not run: it
+ * reports "static staging memory busy" through the failure handler and
+ * returns, leaving its output untouched; the caller may repeat it. The array
+ * keeps the previous call's bytes, and nothing read from it is ever older
+ * than the current call's own uploads. iree_uk_mi355x_init resolves the
+ * array's address ahead of the first call.
+ * Under stream capture itself only the asynchronous mode can be used (a
+ * synchronous call copies and synchronises, which capture forbids), and that
+ * mode takes device operands only: nothing is staged there, and this entry
+ * point then does exactly what iree_uk_mmt4d_p does, which allocates nothing
+ * for device operands either. */
 #define IREE_UK_MI355X_NOALLOC_MAX_STAGED_BYTES (16 * 1024 * 1024)
 void iree_uk_mi355x_mmt4d_noalloc_p(const iree_uk_mmt4d_params_t* params);
 

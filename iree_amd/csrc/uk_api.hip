@@ -107,15 +107,30 @@ constexpr size_t kScratchBytes = (size_t)IREE_UK_MI355X_NOALLOC_MAX_STAGED_BYTES
 constexpr int kMaxDevices = 64;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 std::atomic<unsigned char*> g_scratch_ptr[kMaxDevices];
+// One call at a time may stage host operands in a device's array: taken with a
+// try-lock (a second caller is told so instead of waiting or corrupting the
+// first one's operands), held until the call's results are back on the host.
+std::atomic<bool> g_scratch_busy[kMaxDevices];
+
+struct ScratchLease {
+  std::atomic<bool>* flag = nullptr;
+  ScratchLease() = default;
+  ScratchLease(const ScratchLease&) = delete;
+  ScratchLease& operator=(const ScratchLease&) = delete;
+  ~ScratchLease() {
+    if (flag) flag->store(false, std::memory_order_release);
+  }
+};
 
 // Device address of the current device's `scratch` (nullptr after reporting
 // a failure).
-unsigned char* scratch_for_current_device() {
+unsigned char* scratch_for_current_device(int* device_out = nullptr) {
   int device = -1;
   if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) {
     (void)hipGetLastError();
     return nullptr;
   }
+  if (device_out) *device_out = device;
   unsigned char* ptr = g_scratch_ptr[device].load(std::memory_order_acquire);
   if (ptr) return ptr;
   void* resolved = nullptr;
@@ -135,18 +150,32 @@ struct Stager {
   unsigned char* fixed_base = nullptr;  // non-null: static scratch
   size_t fixed_used = 0;
   bool no_alloc = false;
+  bool copies_issued = false;           // something was enqueued on the stream for this call
+  ScratchLease lease;                   // held while the static scratch is in use
 };
+
+size_t rounded_for_scratch(size_t bytes) { return (bytes + 255) & ~(size_t)255; }
 
 bool stage_reserve(Stager& stager, int slot, size_t bytes, void** out) {
   if (stager.no_alloc) {
     if (!stager.fixed_base) {
-      stager.fixed_base = scratch_for_current_device();
-      if (!stager.fixed_base) {
+      int device = -1;
+      unsigned char* base = scratch_for_current_device(&device);
+      if (!base) {
         report_failure(__FILE__, __LINE__, __func__, "hipGetSymbolAddress(scratch) failed on the current device");
         return false;
       }
+      bool expected = false;
+      if (!g_scratch_busy[device].compare_exchange_strong(expected, true, std::memory_order_acq_rel)) {
+        report_failure(__FILE__, __LINE__, __func__,
+                       "static staging memory busy: another iree_uk_mi355x_mmt4d_noalloc_p call with host "
+                       "operands is running on this device");
+        return false;
+      }
+      stager.lease.flag = &g_scratch_busy[device];
+      stager.fixed_base = base;
     }
-    const size_t rounded = (bytes + 255) & ~(size_t)255;
+    const size_t rounded = rounded_for_scratch(bytes);
     if (rounded > kScratchBytes - stager.fixed_used) {
       report_failure(__FILE__, __LINE__, __func__,
                      "host operands exceed IREE_UK_MI355X_NOALLOC_MAX_STAGED_BYTES of static staging memory");
@@ -235,10 +264,10 @@ struct Staged {
 };
 
 bool stage_operand(Stager& stager, int slot, const void* ptr, const RowRegion& region, bool upload,
-                   hipStream_t stream, Staged* st, const void** dev_ptr) {
+                   hipStream_t stream, Staged* st, const void** dev_ptr, int known_on_device = -1) {
   *dev_ptr = ptr;
   if (region.span == 0) return true;
-  const bool on_device = device_accessible(ptr);
+  const bool on_device = known_on_device < 0 ? device_accessible(ptr) : known_on_device != 0;
   if (tl_async) {
     // Nothing is staged in asynchronous mode, and a host address must not
     // reach a kernel: the device would fault.
@@ -251,7 +280,10 @@ bool stage_operand(Stager& stager, int slot, const void* ptr, const RowRegion& r
   if (on_device) return true;
   void* d = nullptr;
   if (!stage_reserve(stager, slot, (size_t)region.span, &d)) return false;
-  if (upload && !copy_rows(d, ptr, region, hipMemcpyHostToDevice, stream)) return false;
+  if (upload) {
+    stager.copies_issued = true;
+    if (!copy_rows(d, ptr, region, hipMemcpyHostToDevice, stream)) return false;
+  }
   st->host = ptr;
   st->dev = d;
   *dev_ptr = d;
@@ -260,8 +292,10 @@ bool stage_operand(Stager& stager, int slot, const void* ptr, const RowRegion& r
 
 bool finish(hipStream_t stream, const Staged& out, const RowRegion& out_region, bool any_staged) {
   if (out.host && !copy_rows(const_cast<void*>(out.host), out.dev, out_region,
-                             hipMemcpyDeviceToHost, stream))
+                             hipMemcpyDeviceToHost, stream)) {
+    if (!tl_async) (void)hipStreamSynchronize(stream);
     return false;
+  }
   if (!tl_async) UK_HIP_OK(hipStreamSynchronize(stream));
   (void)any_staged;
   return true;
@@ -273,6 +307,13 @@ bool launch_ok(hipError_t e, const char* what) {
   snprintf(msg, sizeof msg, "%s launch -> %s", what, hipGetErrorString(e));
   report_failure(__FILE__, __LINE__, __func__, msg);
   return false;
+}
+
+// Leaves an entry point early after a failure: in synchronous mode nothing
+// of the call may still be in flight when it returns (uploads read the
+// caller's memory, and the staging memory is about to be handed on).
+void abandon(const Stager& stager, hipStream_t stream) {
+  if (!tl_async && stager.copies_issued) (void)hipStreamSynchronize(stream);
 }
 
 uk::Mmt4dLauncher select_mmt4d(const uk::Mmt4dArgs& a, bool probe_only) {
@@ -371,9 +412,31 @@ void mmt4d_impl(const iree_uk_mmt4d_params_t* p, Stager& stager) {
   const void *d_lhs, *d_rhs, *d_out;
   // A host operand whose rows overlap is staged as one span.
   auto as_copied = [](const RowRegion& r) { return r.rows > 1 && r.pitch < r.width ? as_one_span(r) : r; };
-  if (!stage_operand(stager, 0, lhs, as_copied(lhs_region), true, stream, &s_lhs, &d_lhs)) return;
-  if (!stage_operand(stager, 1, rhs, as_copied(rhs_region), true, stream, &s_rhs, &d_rhs)) return;
-  if (!stage_operand(stager, 2, out, out_region, accumulate, stream, &s_out, &d_out)) return;
+  const RowRegion lhs_copy = as_copied(lhs_region), rhs_copy = as_copied(rhs_region);
+  int lhs_dev = -1, rhs_dev = -1, out_dev = -1;
+  if (stager.no_alloc && !tl_async) {
+    // Whether the host operands fit the static memory is settled before the
+    // first byte is copied.
+    lhs_dev = lhs_copy.span == 0 || device_accessible(lhs);
+    rhs_dev = rhs_copy.span == 0 || device_accessible(rhs);
+    out_dev = out_region.span == 0 || device_accessible(out);
+    Checked need;
+    int64_t total = 0;
+    if (!lhs_dev) total = need.add(total, need.add(lhs_copy.span, 255) & ~(int64_t)255);
+    if (!rhs_dev) total = need.add(total, need.add(rhs_copy.span, 255) & ~(int64_t)255);
+    if (!out_dev) total = need.add(total, need.add(out_region.span, 255) & ~(int64_t)255);
+    if (!need.ok || total > (int64_t)kScratchBytes) {
+      report_failure(__FILE__, __LINE__, __func__,
+                     "host operands exceed IREE_UK_MI355X_NOALLOC_MAX_STAGED_BYTES of static staging memory");
+      return;
+    }
+  }
+  if (!stage_operand(stager, 0, lhs, lhs_copy, true, stream, &s_lhs, &d_lhs, lhs_dev) ||
+      !stage_operand(stager, 1, rhs, rhs_copy, true, stream, &s_rhs, &d_rhs, rhs_dev) ||
+      !stage_operand(stager, 2, out, out_region, accumulate, stream, &s_out, &d_out, out_dev)) {
+    abandon(stager, stream);
+    return;
+  }
 
   uk::Mmt4dArgs a;
   a.lhs = (const uint8_t*)d_lhs;
@@ -404,7 +467,10 @@ void mmt4d_impl(const iree_uk_mmt4d_params_t* p, Stager& stager) {
       if (k > 0) part.flags |= IREE_UK_FLAG_MMT4D_ACCUMULATE;
       uk::Mmt4dLauncher launcher = select_mmt4d(part, /*probe_only=*/false);
       if (!launcher) launcher = uk::launch_mmt4d_generic;
-      if (!launch_ok(launcher(part, stream, &tl_last_kernel), "mmt4d")) return;
+      if (!launch_ok(launcher(part, stream, &tl_last_kernel), "mmt4d")) {
+        abandon(stager, stream);
+        return;
+      }
     }
     finish(stream, s_out, out_region, s_lhs.host || s_rhs.host || s_out.host);
     return;
@@ -412,7 +478,10 @@ void mmt4d_impl(const iree_uk_mmt4d_params_t* p, Stager& stager) {
 
   uk::Mmt4dLauncher launcher = select_mmt4d(a, /*probe_only=*/false);
   if (!launcher) launcher = uk::launch_mmt4d_generic;
-  if (!launch_ok(launcher(a, stream, &tl_last_kernel), "mmt4d")) return;
+  if (!launch_ok(launcher(a, stream, &tl_last_kernel), "mmt4d")) {
+    abandon(stager, stream);
+    return;
+  }
   finish(stream, s_out, out_region, s_lhs.host || s_rhs.host || s_out.host);
 }
 
@@ -521,8 +590,11 @@ UK_API void iree_uk_pack_p(const iree_uk_pack_params_t* p) {
   RowRegion in_copy = in_region;
   if (in_copy.rows > 1 && in_copy.pitch < in_copy.width) in_copy = as_one_span(in_region);
   Stager stager;
-  if (!stage_operand(stager, 0, in, in_copy, true, stream, &s_in, &d_in)) return;
-  if (!stage_operand(stager, 2, out, out_region, false, stream, &s_out, &d_out)) return;
+  if (!stage_operand(stager, 0, in, in_copy, true, stream, &s_in, &d_in) ||
+      !stage_operand(stager, 2, out, out_region, false, stream, &s_out, &d_out)) {
+    abandon(stager, stream);
+    return;
+  }
 
   uk::PackArgs a;
   a.in = (const uint8_t*)d_in;
@@ -535,7 +607,10 @@ UK_API void iree_uk_pack_p(const iree_uk_pack_params_t* p) {
   a.padding_value = p->padding_value;
   a.flags = p->flags;
   a.elem_bytes = e;
-  if (!launch_ok(uk::launch_pack(a, stream, &tl_last_kernel), "pack")) return;
+  if (!launch_ok(uk::launch_pack(a, stream, &tl_last_kernel), "pack")) {
+    abandon(stager, stream);
+    return;
+  }
   finish(stream, s_out, out_region, s_in.host || s_out.host);
 }
 
@@ -609,10 +684,13 @@ UK_API void iree_uk_unpack_p(const iree_uk_unpack_params_t* p) {
   Staged s_in, s_out;
   const void *d_in, *d_out;
   Stager stager;
-  if (!stage_operand(stager, 0, in, in_region, true, stream, &s_in, &d_in)) return;
   // With an inner output stride the bytes between elements must survive the
   // round trip through the staging buffer, so the rows are uploaded first.
-  if (!stage_operand(stager, 2, out, out_region, p->out_stride1 != 1, stream, &s_out, &d_out)) return;
+  if (!stage_operand(stager, 0, in, in_region, true, stream, &s_in, &d_in) ||
+      !stage_operand(stager, 2, out, out_region, p->out_stride1 != 1, stream, &s_out, &d_out)) {
+    abandon(stager, stream);
+    return;
+  }
 
   uk::UnpackArgs a;
   a.in = (const uint8_t*)d_in;
@@ -624,7 +702,10 @@ UK_API void iree_uk_unpack_p(const iree_uk_unpack_params_t* p) {
   a.out_size0 = p->out_size0; a.out_size1 = p->out_size1;
   a.flags = p->flags;
   a.elem_bytes = e;
-  if (!launch_ok(uk::launch_unpack(a, stream, &tl_last_kernel), "unpack")) return;
+  if (!launch_ok(uk::launch_unpack(a, stream, &tl_last_kernel), "unpack")) {
+    abandon(stager, stream);
+    return;
+  }
   finish(stream, s_out, out_region, s_in.host || s_out.host);
 }
 

@@ -119,3 +119,114 @@ def test_noalloc_rejects_operands_beyond_its_static_memory():
     # The same shapes still run on the allocating entry point.
     lib.iree_uk_mmt4d_p(C.byref(_params(lhs, rhs, out, M, N, K, M0, N0, K0, abi.MMT4D_TYPE_S8S8S32)))
     assert np.all(out == 0)
+
+
+def _run_in_thread(fn):
+    import threading
+    box = {}
+
+    def body():
+        try:
+            box["value"] = fn()
+        except BaseException as e:   # re-raised in the caller
+            box["error"] = e
+    t = threading.Thread(target=body)
+    t.start()
+    t.join()
+    if "error" in box:
+        raise box["error"]
+    return box.get("value")
+
+
+def test_noalloc_call_leaves_free_device_memory_unchanged():
+    """The property the entry point exists for: no hipMalloc / hipFree. A fresh host thread owns no staging
+    buffers, so its first call with host operands is where the allocating entry point must allocate
+    (seen below as a drop in free device memory, which shows that the measure can see it) and where this one
+    must not."""
+    lib = library.load()
+    assert lib.iree_uk_mi355x_init(0) == 0
+    lib.iree_uk_mi355x_set_stream(None, 0)
+    M, N, K, M0, N0, K0 = 96, 64, 512, 8, 8, 4     # lhs 1.5 MiB, rhs 1 MiB, out 1.5 MiB of host memory
+    flags = abi.MMT4D_TYPE_S8S8S32
+    lhs, rhs, init, _, _ = _case(11, M, N, K, M0, N0, K0, flags)
+    torch.cuda.synchronize()
+
+    def measure(entry):
+        def body():
+            assert lib.iree_uk_mi355x_init(0) == 0
+            out = init.copy()
+            free_before, _ = torch.cuda.mem_get_info()
+            entry(C.byref(_params(lhs, rhs, out, M, N, K, M0, N0, K0, flags)))
+            free_after, _ = torch.cuda.mem_get_info()
+            return free_before - free_after, out
+        return _run_in_thread(body)
+
+    used_noalloc, got = measure(lib.iree_uk_mi355x_mmt4d_noalloc_p)
+    used_alloc, want = measure(lib.iree_uk_mmt4d_p)
+    assert np.array_equal(got, want)
+    assert used_noalloc == 0, used_noalloc
+    assert used_alloc >= lhs.nbytes + rhs.nbytes + init.nbytes, used_alloc
+
+
+def test_noalloc_overlapping_calls_are_correct_or_cleanly_refused():
+    """Two host threads call the entry point with host operands at the same time, on one device: they share
+    its static staging memory, which only one call may use at a time. Every call must either produce the
+    result of the allocating entry point or be refused through the failure handler with its output
+    untouched ("static staging memory busy"); the microkernels are to be callable from many threads
+    (the reference's README.md:26)."""
+    import threading
+    lib = library.load()
+    assert lib.iree_uk_mi355x_init(0) == 0
+    lib.iree_uk_mi355x_set_stream(None, 0)
+    M, N, K, M0, N0, K0 = 64, 48, 512, 8, 8, 4
+    flags = abi.MMT4D_TYPE_S8S8S32 | abi.MMT4D_ACCUMULATE
+    cases = []
+    for seed in (31, 32):
+        lhs, rhs, init, _, _ = _case(seed, M, N, K, M0, N0, K0, flags)
+        want = init.copy()
+        lib.iree_uk_mmt4d_p(C.byref(_params(lhs, rhs, want, M, N, K, M0, N0, K0, flags)))
+        cases.append((lhs, rhs, init, want))
+
+    refused = {}    # thread id -> messages
+    cb = library.FAIL_HANDLER(lambda f, l, fn, cond: refused.setdefault(threading.get_ident(), []).append(cond.decode()))
+    lib.iree_uk_mi355x_set_fail_handler(cb)
+    outcomes = {0: [0, 0], 1: [0, 0]}   # worker -> [done, refused]
+    errors = []
+    start = threading.Barrier(2)
+
+    def worker(w):
+        try:
+            assert lib.iree_uk_mi355x_init(0) == 0
+            lhs, rhs, init, want = cases[w]
+            mine = refused.setdefault(threading.get_ident(), [])
+            start.wait()
+            for _ in range(60):
+                out = init.copy()
+                before = len(mine)
+                lib.iree_uk_mi355x_mmt4d_noalloc_p(C.byref(_params(lhs, rhs, out, M, N, K, M0, N0, K0, flags)))
+                if len(mine) > before:
+                    assert len(mine) == before + 1 and "static staging memory busy" in mine[-1], mine[-1]
+                    assert np.array_equal(out, init), "a refused call wrote its output"
+                    outcomes[w][1] += 1
+                else:
+                    assert np.array_equal(out, want), "an accepted call gave a wrong result"
+                    outcomes[w][0] += 1
+        except BaseException as e:
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(w,)) for w in (0, 1)]
+    try:
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+    finally:
+        lib.iree_uk_mi355x_set_fail_handler(library.FAIL_HANDLER(0))
+    if errors:
+        raise errors[0]
+    assert outcomes[0][0] > 0 and outcomes[1][0] > 0, outcomes
+    assert sum(outcomes[0]) == 60 and sum(outcomes[1]) == 60, outcomes
+    # Afterwards the memory is free again.
+    out = cases[0][2].copy()
+    lib.iree_uk_mi355x_mmt4d_noalloc_p(C.byref(_params(cases[0][0], cases[0][1], out, M, N, K, M0, N0, K0, flags)))
+    assert np.array_equal(out, cases[0][3])
