@@ -149,6 +149,111 @@ __global__ __launch_bounds__(64 * kWaves) void mmt4d_gemv_kernel(const GemvArgs 
   }
 }
 
+// The same product for more than 4 lhs rows, where the lhs operand of a K-step
+// is as large as a rhs tile's (1 KiB) and the kernel above pulls all of it
+// through L2 again for every rhs tile. Here one workgroup per compute unit
+// stays for the whole launch: its wavefronts split K, wavefront w copies the lhs
+// operands of its K share into a private slice of LDS once, and then streams
+// the rhs tiles of the unit's range past them, the loads of the next tile in
+// flight while the current one is multiplied. No barrier before the final sum.
+// The rhs is dealt out in HALF tiles (rhs rows 0-7 or 8-15 of a tile: 128
+// contiguous bytes of every k step for 16-byte row pieces) so that every unit
+// gets the same number of bytes also when tiles / units is not whole (896 tiles
+// on 256 units: 3.5); a half tile is a tile with half the lanes' loads masked,
+// its missing rows multiply as zeros and are not stored. Partial sums meet in
+// LDS in wavefront order: results do not depend on scheduling.
+// Needs steps == kWaves * UNROLL (one batch of loads per wavefront and tile).
+template <int KIND, int kWaves, int UNROLL, int MAX_TILES>
+__global__ __launch_bounds__(64 * kWaves) void mmt4d_gemv_resident_lhs_kernel(const GemvArgs a) {
+  typedef typename Acc<KIND>::type acc_t;
+  extern __shared__ uint4 gemv_lds[];  // [kWaves][UNROLL][64] lhs operands; then [MAX_TILES][kWaves][64] partial sums
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int row = lane & 15, g = lane >> 4;
+  const int32_t M0 = 1 << a.log2_M0;
+  const int32_t lhs_rows = a.M << a.log2_M0;  // <= 16
+
+  // This unit's range of half tiles.
+  const int64_t halves = 2 * (int64_t)a.N;
+  const int64_t h0 = (int64_t)blockIdx.x * halves / gridDim.x, h1 = ((int64_t)blockIdx.x + 1) * halves / gridDim.x;
+  if (h1 <= h0) return;
+  const int64_t t0 = h0 >> 1, t1 = (h1 - 1) >> 1;
+  const int tiles = (int)(t1 - t0 + 1);  // <= MAX_TILES (checked on the host)
+  const bool skip_low_half_of_first = h0 & 1, skip_high_half_of_last = h1 & 1;
+
+  const int32_t ksteps_per_step = 64 >> a.log2_rb;
+  const int32_t k1_lane = (16 * g) >> a.log2_rb;
+  const int32_t within = (16 * g) & (a.rb - 1);
+  const int64_t rhs_kstep = (int64_t)a.rb * 16;
+  const int64_t lhs_kstep = (int64_t)a.rb << a.log2_M0;
+  const bool lhs_valid = row < lhs_rows;
+  const int64_t k1_first = (int64_t)(wave * UNROLL) * ksteps_per_step;  // this wavefront's share of K
+  const uint8_t* lhs_lane = a.lhs + (int64_t)(row >> a.log2_M0) * a.lhs_stride_bytes +
+                            (int64_t)(row & (M0 - 1)) * a.rb + (k1_lane + k1_first) * lhs_kstep + within;
+  const uint8_t* rhs_lane = a.rhs + t0 * a.rhs_stride_bytes + (int64_t)row * a.rb +
+                            (k1_lane + k1_first) * rhs_kstep + within;
+  const int64_t rhs_step_bytes = ksteps_per_step * rhs_kstep, lhs_step_bytes = ksteps_per_step * lhs_kstep;
+
+  auto tile_rows_loaded = [&](int u) -> bool {
+    if (u == 0 && skip_low_half_of_first && row < 8) return false;
+    if (u == tiles - 1 && skip_high_half_of_last && row >= 8) return false;
+    return true;
+  };
+  uint4 r[2][UNROLL];
+  auto fetch = [&](int u, uint4* dst) {
+    const uint8_t* p = rhs_lane + (int64_t)u * a.rhs_stride_bytes;
+    const bool loaded = tile_rows_loaded(u);
+#pragma unroll
+    for (int s = 0; s < UNROLL; ++s) {
+      dst[s] = make_uint4(0, 0, 0, 0);
+      if (loaded) dst[s] = __builtin_bit_cast(uint4, __builtin_nontemporal_load((const v4i32*)(p + s * rhs_step_bytes)));
+    }
+  };
+  fetch(0, r[0]);
+  uint4* own_lhs = gemv_lds + (wave * UNROLL) * 64 + lane;
+  {
+    uint4 l[UNROLL];
+#pragma unroll
+    for (int s = 0; s < UNROLL; ++s) {
+      l[s] = make_uint4(0, 0, 0, 0);
+      if (lhs_valid) l[s] = *(const uint4*)(lhs_lane + s * lhs_step_bytes);
+    }
+#pragma unroll
+    for (int s = 0; s < UNROLL; ++s) own_lhs[s * 64] = l[s];
+  }
+
+  acc_t acc[MAX_TILES];
+#pragma unroll
+  for (int u = 0; u < MAX_TILES; ++u) acc[u] = acc_t{0, 0, 0, 0};
+#pragma unroll
+  for (int u = 0; u < MAX_TILES; ++u) {
+    if (u < tiles) {
+      if (u + 1 < tiles) fetch(u + 1, r[(u + 1) & 1]);
+#pragma unroll
+      for (int s = 0; s < UNROLL; ++s) acc[u] = mfma16<KIND>(r[u & 1][s], own_lhs[s * 64], acc[u]);
+    }
+  }
+
+  __syncthreads();  // the lhs slices are no longer read: their memory takes the partial sums
+  acc_t* partial = (acc_t*)gemv_lds;
+#pragma unroll
+  for (int u = 0; u < MAX_TILES; ++u)
+    if (u < tiles) partial[(u * kWaves + wave) * 64 + lane] = acc[u];
+  __syncthreads();
+  // Lane l holds lhs row l & 15 and rhs rows 4*(l >> 4) + {0..3} of each tile: four consecutive j0 of output row i0.
+  for (int u = wave; u < tiles; u += kWaves) {
+    if (!lhs_valid) continue;
+    if (u == 0 && skip_low_half_of_first && g < 2) continue;
+    if (u == tiles - 1 && skip_high_half_of_last && g >= 2) continue;
+    acc_t v = partial[(u * kWaves) * 64 + lane];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) v += partial[(u * kWaves + w) * 64 + lane];
+    acc_t* dst = (acc_t*)(a.out + 4 * ((int64_t)(row >> a.log2_M0) * a.out_stride0 + (t0 + u) * ((int64_t)M0 * 16) +
+                                       (int64_t)(row & (M0 - 1)) * 16 + 4 * g));
+    if (a.accumulate) v += *dst;
+    *dst = v;
+  }
+}
+
 // int8 values equal to 16x the signed nibbles of 8 bytes, in element order
 // (element 2b in the low nibble of byte b, mmt4d_tile_generic.c:35-45): even
 // and odd elements are isolated in the high nibbles of two dwords whose bytes
@@ -305,8 +410,54 @@ bool make_args(const Mmt4dArgs& a, bool probe_only, int* kind, GemvArgs* g) {
   return true;
 }
 
+// Compute units of the current device (one persistent workgroup each).
+int compute_units() {
+  static int cached[64] = {0};
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 0;
+  if (cached[device] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return 0;
+    cached[device] = n;
+  }
+  return cached[device];
+}
+
+// The resident-lhs kernel, if it fits: more than 4 lhs rows, K in whole 64-byte
+// steps whose number is what one of the instantiations splits over its
+// wavefronts, at least a tile per compute unit and at most MAX_TILES of them.
 template <int KIND>
-hipError_t launch_kind(const GemvArgs& g, hipStream_t stream) {
+bool launch_resident_lhs(const GemvArgs& g, hipStream_t stream, hipError_t* status) {
+  constexpr int MAX_TILES = 8;
+  // (With 1 or 4 lhs rows the kernel above is the faster one: 6.14 against 6.0 TB/s at 896 tiles.)
+  if ((g.M << g.log2_M0) <= 4) return false;
+  if (((int64_t)g.K * g.rb) % 64 != 0) return false;
+  const int units = compute_units();
+  if (units <= 0 || g.N < units) return false;
+  // (most tiles any unit gets: ceil(2N / units) half tiles can touch that many / 2 + 1 tiles)
+  if ((2 * (int64_t)g.N + units - 1) / units / 2 + 1 > MAX_TILES) return false;
+  auto launch = [&](auto kernel, int waves, int unroll) {
+    const int lds_bytes = waves * (unroll > MAX_TILES ? unroll : MAX_TILES) * 1024;
+    *status = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (*status != hipSuccess) return;
+    hipLaunchKernelGGL(kernel, dim3(units), dim3(64 * waves), lds_bytes, stream, g);
+    *status = hipGetLastError();
+  };
+  // (8 wavefronts with 16 loads each in flight twice over; 16 wavefronts x 8 measured no better than the kernel above.)
+  switch (g.steps) {
+    case 128: launch(mmt4d_gemv_resident_lhs_kernel<KIND, 8, 16, MAX_TILES>, 8, 16); return true;
+    case 64: launch(mmt4d_gemv_resident_lhs_kernel<KIND, 8, 8, MAX_TILES>, 8, 8); return true;
+    default: return false;
+  }
+}
+
+template <int KIND>
+hipError_t launch_kind(const GemvArgs& g, hipStream_t stream, const char** name) {
+  hipError_t status;
+  if (launch_resident_lhs<KIND>(g, stream, &status)) {
+    *name = "mmt4d_gemv_resident_lhs";
+    return status;
+  }
   // One rhs tile per workgroup (most workgroups, best balance over the CUs),
   // 4 wavefronts splitting K, 16 KiB of rhs in flight per wavefront.
   constexpr int TN = 1, UNROLL = 16, WAVES = 4;
@@ -330,9 +481,9 @@ hipError_t launch_gemv(const Mmt4dArgs& a, hipStream_t stream, const char** name
     }
     return hipGetLastError();
   }
-  if (kind == kI8) return launch_kind<kI8>(g, stream);
-  if (kind == kF16) return launch_kind<kF16>(g, stream);
-  return launch_kind<kBF16>(g, stream);
+  if (kind == kI8) return launch_kind<kI8>(g, stream, name);
+  if (kind == kF16) return launch_kind<kF16>(g, stream, name);
+  return launch_kind<kBF16>(g, stream, name);
 }
 
 }  // namespace

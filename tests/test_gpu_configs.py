@@ -208,7 +208,7 @@ def test_bf16_skinny_decode_shapes(gpu_lib, oracle_lib, m0):
     d_o = torch.full((N * m0 * N0,), 7.0, dtype=torch.float32, device="cuda")
     q = mm_params(d_l.data_ptr(), d_r.data_ptr(), d_o.data_ptr(), 1, N, K, m0, N0, K0, flags)
     gpu_lib.iree_uk_mmt4d_p(C.byref(q))
-    assert gpu_lib.iree_uk_mi355x_last_kernel() == b"mmt4d_gemv"
+    assert gpu_lib.iree_uk_mi355x_last_kernel() == (b"mmt4d_gemv_resident_lhs" if m0 == 16 else b"mmt4d_gemv")
     assert_float_close(d_o.cpu().numpy(), want, "bf16 skinny M0=%d" % m0)
     # accumulate: out += product, starting from a known buffer
     start = synth.normal_f32(4, 99, N * m0 * N0, 1.0)

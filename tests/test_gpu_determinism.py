@@ -27,6 +27,7 @@ CASES = [
     (abi.MMT4D_TYPE_F16F16F16 | SKIP, 16, 16, 64, 16, 16, 16, b"mmt4d_mfma_"),
     (BF16, 1, 100, 300, 16, 16, 8, b"mmt4d_gemv"),
     (F16, 1, 77, 1000, 4, 16, 8, b"mmt4d_gemv"),
+    (BF16, 1, 333, 512, 16, 16, 8, b"mmt4d_gemv_resident_lhs"),
     (F16, 1, 50, 3000, 1, 16, 1, b"mmt4d_skinny"),
     (BF16, 1, 40, 2000, 4, 16, 2, b"mmt4d_skinny"),
     (F32, 1, 60, 1500, 2, 8, 1, b"mmt4d_skinny"),

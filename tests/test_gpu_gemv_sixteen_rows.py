@@ -84,3 +84,65 @@ def test_tile_counts_around_the_number_of_compute_units(gpu_lib, oracle_lib, N, 
     got = d_all.cpu().numpy()
     assert np.array_equal(got[64:-64], want)
     assert (got[:64] == 123456).all() and (got[-64:] == 123456).all()
+
+
+# The resident-lhs kernel (one workgroup per compute unit, the lhs operands of each wavefront's K share copied to
+# LDS once, rhs dealt out in half tiles): at least one rhs tile per compute unit, more than 4 lhs rows, K of
+# 64 or 128 steps of 64 bytes. Tile counts that give the units whole tiles, half tiles at either end of their
+# ranges, and ranges of unequal length; lhs rows from one, two and four lhs tiles, fewer than 16 rows; a gap
+# between rhs panels, strided lhs and out rows; with guard words around the output. int8 bit for bit.
+RESIDENT = [
+    # flags, M, M0, N, K, K0
+    (abi.MMT4D_TYPE_S8S8S32, 1, 16, 896, 64, 64),     # 64 steps; 3.5 tiles per unit
+    (abi.MMT4D_TYPE_S8S8S32, 1, 16, 256, 128, 64),    # 128 steps; exactly one tile per unit
+    (abi.MMT4D_TYPE_S8S8S32, 2, 8, 257, 256, 16),     # 64 steps; two lhs tiles of 8 rows
+    (abi.MMT4D_TYPE_S8S8S32, 4, 4, 1000, 128, 32),    # 64 steps; four lhs tiles of 4 rows
+    (abi.MMT4D_TYPE_S8S8S32, 3, 4, 511, 512, 16),     # 128 steps; 12 lhs rows
+    (abi.MMT4D_TYPE_S8S8S32, 1, 8, 1791, 64, 64),     # 8 lhs rows; 7 tiles per unit at most
+    (abi.MMT4D_TYPE_BF16BF16F32, 1, 16, 897, 512, 8),   # the decode shape plus one tile
+    (abi.MMT4D_TYPE_F16F16F32, 1, 16, 300, 128, 16),    # rb 32, 64 steps
+    (abi.MMT4D_TYPE_BF16BF16F32, 2, 8, 384, 256, 16),   # rb 32, 128 steps
+]
+
+
+@pytest.mark.parametrize("case", RESIDENT, ids=lambda c: "t%x_M%dx%d_N%d_K%d_K0%d" % c)
+@pytest.mark.parametrize("acc", [0, abi.MMT4D_ACCUMULATE])
+def test_resident_lhs_kernel(gpu_lib, oracle_lib, case, acc):
+    flags, M, M0, N, K, K0 = case
+    N0 = 16
+    flags |= acc
+    lhs_stride, rhs_stride, out_stride = K * M0 * K0 + 32, K * N0 * K0 + 64, N * M0 * N0 + 8
+    if (flags & 0xFF) == abi.MMT4D_TYPE_S8S8S32:
+        lhs = synth.uniform_int8(47, 0, M * lhs_stride)
+        rhs = synth.uniform_int8(47, 1, N * rhs_stride)
+        init = (synth.uniform_int8(47, 2, M * out_stride).astype(np.int32)) * 1000
+    else:
+        to_bits = synth.f16_bits if (flags & 0xFF) == abi.MMT4D_TYPE_F16F16F32 else synth.bf16_bits
+        lhs = to_bits(synth.normal_f32(47, 0, M * lhs_stride, 1.0))
+        rhs = to_bits(synth.normal_f32(47, 1, N * rhs_stride, 0.05))
+        init = synth.normal_f32(47, 2, M * out_stride, 1.0)
+
+    def strided(p):
+        p.lhs_stride0, p.rhs_stride0, p.out_stride0 = lhs_stride, rhs_stride, out_stride
+        return p
+    want = init.copy()
+    oracle_lib.oracle_mmt4d_mt(C.byref(strided(mm_params(lhs.ctypes.data, rhs.ctypes.data, want.ctypes.data, M, N, K,
+                                                         M0, N0, K0, flags | abi.MMT4D_ALLOW_GENERIC_FALLBACK))), 8)
+    as_dev = lambda x: torch.from_numpy(x.view(np.int16) if x.dtype == np.uint16 else x).cuda()
+    d_l, d_r = as_dev(lhs), as_dev(rhs)
+    guard = torch.full((64,), 7, dtype=torch.from_numpy(init).dtype, device="cuda")
+    d_all = torch.cat([guard, torch.from_numpy(init.copy()).cuda(), guard])
+    gpu_lib.iree_uk_mmt4d_p(C.byref(strided(mm_params(d_l.data_ptr(), d_r.data_ptr(), d_all.data_ptr() + 256, M, N, K,
+                                                      M0, N0, K0, flags))))
+    assert gpu_lib.iree_uk_mi355x_last_kernel() == b"mmt4d_gemv_resident_lhs"
+    got_all = d_all.cpu().numpy()
+    got = got_all[64:-64]
+    assert (got_all[:64] == 7).all() and (got_all[-64:] == 7).all()
+    if want.dtype == np.int32:
+        assert np.array_equal(got, want)       # the gaps between out rows included
+    else:
+        rows = np.arange(M * out_stride).reshape(M, out_stride)
+        inside = rows[:, :N * M0 * N0].reshape(-1)
+        assert_float_close(got[inside], want[inside], "resident lhs %r" % (case,))
+        gaps = rows[:, N * M0 * N0:].reshape(-1)
+        assert np.array_equal(got[gaps], init[gaps])
