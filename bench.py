@@ -107,6 +107,24 @@ def _headline(torch, lib, abi, synth, steps, warmup):
                          "accumulate off, operands resident in HBM")
 
 
+def _sustained_ceiling(torch, abi, synth):
+    """What the matrix pipe sustains on the headline's data with the headline kernel's inner-loop instruction
+    mix (32 MFMAs, 16 LDS reads, 8 loads to LDS, one barrier per step) and no HBM traffic, prologue or
+    epilogue: the benchmark's probe on uniformly random int8. The published peak assumes 2.4 GHz; the part
+    clocks lower on data that toggles."""
+    from iree_amd import library
+    rnd = torch.from_numpy(synth.uniform_int8(0, 0, 2 << 20)).cuda()
+    tops, mhz = C.c_double(), C.c_double()
+    rc = library.load_bench_probe().uk_bench_probe_matrix_pipe(abi.MMT4D_TYPE_S8S8S32, rnd.data_ptr(), rnd.numel(), 1, 4096,
+                                                               C.byref(tops), C.byref(mhz))
+    if rc != 0:
+        raise RuntimeError("matrix pipe probe failed: HIP error %d" % rc)
+    return {"value": round(tops.value, 1), "unit": "TOP/s", "shader_mhz": round(mhz.value),
+            "frac_of_peak": round(tops.value / PEAK_INT8_TOPS, 4),
+            "what": "probe: the kernel's MFMA + LDS instruction mix on uniformly random int8, L1-resident operands, "
+                    "no prologue, no store"}
+
+
 def _e2e_chain(torch, lib, abi, synth, steps, warmup):
     """The chain the reference's matmul benchmark runs (tools/e2e_matmul_benchmark.c:173-186):
     pack lhs, pack rhs (given as [K, N], both transposes), mmt4d, unpack, on row-major int8
@@ -515,6 +533,37 @@ def _also(torch, lib, abi, synth, steps, warmup):
         "what": "torch.Tensor.copy_ of the same matrix (read + write counted)", "ms": round(ms, 5),
         "value": round(2 * R * Cc * 4 / ms / 1e6, 1), "unit": "GB/s",
         "frac_of_peak": round(2 * R * Cc * 4 / ms / 1e6 / PEAK_HBM_GBS, 4)}
+    # What the device streams with plain kernels and nothing else to do (the
+    # benchmark's own probe, csrc/bench/probe_hbm_stream.hip: 16 bytes per lane, read
+    # only / write only / copy, best of a few launch shapes), over the same two
+    # buffer sets. The GB/s rows of this library are reported against these as well
+    # (`of_stream_ceiling`): against the copy for pack and unpack, against the
+    # read-only stream for the matrix-vector kernels.
+    probe_lib = library.load_bench_probe()
+    sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+    stream_bytes = R * Cc * 4 // 16 * 16
+    ceilings = {}
+    for mode, mode_name in ((0, "read_only"), (1, "write_only"), (2, "copy")):
+        best = None
+        for unroll, grid in ((4, 0), (8, 0), (4, 4096), (8, 2048)):
+            st = {"i": 0}
+
+            def stream_step():
+                i = st["i"] & 1
+                rc = probe_lib.uk_bench_probe_hbm_stream(mode, back[i].data_ptr(), src[i].data_ptr(), stream_bytes, grid,
+                                                         unroll, 1, sink.data_ptr(),
+                                                         torch.cuda.current_stream().cuda_stream)
+                if rc != 0:
+                    raise RuntimeError("hbm stream probe failed: HIP error %d" % rc)
+                st["i"] += 1
+            ms, _ = _time_launches(torch, stream_step, max(steps, 6), warmup)
+            best = ms if best is None else min(best, ms)
+        moved = stream_bytes * (2 if mode == 2 else 1)
+        ceilings[mode_name] = {"ms": round(best, 5), "value": round(moved / best / 1e6, 1), "unit": "GB/s",
+                               "frac_of_peak": round(moved / best / 1e6 / PEAK_HBM_GBS, 4)}
+    res["hbm_stream_ceiling"] = dict(
+        ceilings, what="plain read / fill / copy kernels over %d bytes, non-temporal 16-byte accesses, "
+                       "two buffer sets rotated; best of four launch shapes each" % stream_bytes)
     del src, packed, back
 
     # int8 operands of a 16384^3 matmul into the layouts of the 16x16x64 tile:
@@ -555,6 +604,11 @@ def _also(torch, lib, abi, synth, steps, warmup):
     lib.iree_uk_pack_p(C.byref(pack_i8(0, abi.PACK_TRANSPOSE_INNER | abi.PACK_TRANSPOSE_OUTER, 16, 64)))
     torch.cuda.synchronize()
     res["pack_i8_rhs_layout_bit_exact"] = bool(torch.equal(want, idst[0]))
+    for name, entry in res.items():
+        if isinstance(entry, dict) and entry.get("unit") == "GB/s" and "kernel" in entry:
+            against = "copy" if name.startswith(("pack_", "unpack_")) else "read_only"
+            entry["of_stream_ceiling"] = round(entry["value"] / ceilings[against]["value"], 4)
+            entry["stream_ceiling"] = against
     return res
 
 
@@ -836,6 +890,7 @@ def main():
     lib.iree_uk_mi355x_set_stream(torch.cuda.current_stream().cuda_stream, 1)
 
     head = _headline(torch, lib, abi, synth, args.steps, args.warmup)
+    sustained = _sustained_ceiling(torch, abi, synth)
     also = None if args.no_also else _also(torch, lib, abi, synth, max(6, args.steps // 5), 2)
     lib.iree_uk_mi355x_set_stream(None, 0)
     if also is not None:
@@ -883,7 +938,10 @@ def main():
                      "kernel_ms_mean_back_to_back": round(head["ev_ms"], 5),
                      # Each launch between its own pair of events (includes the events' own gaps).
                      "kernel_ms_single_launch_median": round(head["med_ms"], 5),
-                     "kernel_ms_single_launch_min": round(head["min_ms"], 5)},
+                     "kernel_ms_single_launch_min": round(head["min_ms"], 5),
+                     # Not the roofline: what the instruction mix sustains on this data at the clock the
+                     # part grants it, and `achieved` as a fraction of that.
+                     "sustained_ceiling": dict(sustained, achieved_of_it=round(tops / sustained["value"], 4))},
         "cpu_baseline": cpu,
     }
     if cpu_arch is not None:

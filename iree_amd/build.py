@@ -94,9 +94,10 @@ def build(verbose=False, jobs=8):
 
 
 def build_bench_probe():
-    """The matrix-pipe probe bench.py reports next to the mmt4d figures."""
-    cmd = [HIPCC] + COMMON_FLAGS + ["-shared", os.path.join(CSRC, "bench", "probe_matrix_pipe.hip"),
-                                    "-o", BENCH_PROBE_PATH]
+    """The matrix-pipe and HBM-stream probes bench.py reports next to its figures."""
+    bench_dir = os.path.join(CSRC, "bench")
+    cmd = [HIPCC] + COMMON_FLAGS + ["-shared"] + sorted(
+        os.path.join(bench_dir, f) for f in os.listdir(bench_dir) if f.endswith(".hip")) + ["-o", BENCH_PROBE_PATH]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
         raise RuntimeError("bench probe build failed:\n" + r.stdout)

@@ -68,9 +68,10 @@ _bench_probe = None
 
 
 def load_bench_probe():
-    """The benchmark's matrix-pipe probe (csrc/bench/probe_matrix_pipe.hip), a
-    helper library of its own: what the matrix pipe sustains on given operand
-    bytes. Not part of the microkernel ABI."""
+    """The benchmark's probes (csrc/bench/), a helper library of its own: what the
+    matrix pipe sustains on given operand bytes, and what the device streams to
+    and from HBM with plain read, fill and copy kernels. Not part of the
+    microkernel ABI."""
     global _bench_probe
     if _bench_probe is None:
         path = os.path.join(HERE, "libuk_bench_probe.so")
@@ -80,5 +81,8 @@ def load_bench_probe():
         l.uk_bench_probe_matrix_pipe.argtypes = [C.c_uint32, C.c_void_p, C.c_longlong, C.c_int, C.c_int,
                                                  C.POINTER(C.c_double), C.POINTER(C.c_double)]
         l.uk_bench_probe_matrix_pipe.restype = C.c_int
+        l.uk_bench_probe_hbm_stream.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_longlong, C.c_int, C.c_int,
+                                                C.c_int, C.c_void_p, C.c_void_p]
+        l.uk_bench_probe_hbm_stream.restype = C.c_int
         _bench_probe = l
     return _bench_probe
