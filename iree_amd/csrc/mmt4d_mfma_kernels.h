@@ -591,6 +591,15 @@ __device__ __forceinline__ uint2 lds_read_transposed(const uint8_t* p) {
   return make_uint2((uint32_t)v.x, (uint32_t)v.y);
 }
 
+// A wavefront-uniform pointer, said to be so: the loads above take their base from scalar registers, and whether
+// the compiler keeps a uniform 64-bit address computation on the scalar unit depends on what else uses its inputs.
+__device__ __forceinline__ const uint8_t* uniform_pointer(const uint8_t* p) {
+  const uint64_t v = (uint64_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return (const uint8_t*)(((uint64_t)hi << 32) | lo);
+}
+
 template <int N>
 __device__ __forceinline__ void wait_loads_but() {
   static_assert(N >= 0 && N <= 63, "vmcnt is a 6-bit counter");
@@ -600,7 +609,9 @@ __device__ __forceinline__ void wait_loads_but() {
 // (The 256x256 tile needs all 512 registers of a lane for one wavefront; said
 // explicitly, because left to its occupancy heuristics the compiler may keep
 // the accumulators in scratch memory instead.)
-template <int KIND, bool RHS_I4, bool NARROW, int G, int AM, int BN, int STAGES>
+// STAGGER: 0 = every accumulator stored after the last MFMA; 1 = staggered tail (see below); 2 = the same for
+// an accumulating call.
+template <int KIND, bool RHS_I4, bool NARROW, int G, int AM, int BN, int STAGES, int STAGGER = 0>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, AM * BN >= 16 ? 1 : (AM * BN >= 4 ? 2 : 4))))
 void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   typedef typename AccType<KIND>::type acc_t;
@@ -639,8 +650,8 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
 
   const int64_t first_row = (int64_t)tile_row * BLOCK_ROWS;
   const int64_t first_col = (int64_t)tile_col * BLOCK_COLS;
-  const uint8_t* lhs_base = a.lhs + (first_row >> a.log2_M0) * a.lhs_stride_bytes;
-  const uint8_t* rhs_base = a.rhs + (first_col >> a.log2_N0) * a.rhs_stride_bytes;
+  const uint8_t* lhs_base = uniform_pointer(a.lhs + (first_row >> a.log2_M0) * a.lhs_stride_bytes);
+  const uint8_t* rhs_base = uniform_pointer(a.rhs + (first_col >> a.log2_N0) * a.rhs_stride_bytes);
 
   // Load t of wavefront w fills the 16-byte LDS slots 64*m .. 64*m + 63 of its
   // operand, m = 4*t + w, lane l the slot 64*m + l.
@@ -1102,6 +1113,214 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
     }
   };
 
+  // The last AHEAD chunks, for the 256x256 tile. At the end of the loop above
+  // every accumulator becomes final at the same moment, and the whole tile (256
+  // KiB per workgroup, the whole output of the launch in one burst) is stored
+  // with the matrix pipe idle. Here the loop stops AHEAD chunks early, when
+  // their operands are all in the workgroup already (one chunk's fragments in
+  // registers, the others in the ring), and those chunks are multiplied in
+  // another order: first the register chunk as usual, during which the loads
+  // still in flight are awaited and the ring chunks' rhs fragments and the first
+  // row's lhs fragments are read; then fragment by fragment, two fragments of a
+  // row at a time, each pair running through the ring chunks and being stored
+  // while the next pair is multiplied (one 128-bit store per MFMA, the first
+  // behind the pair's last MFMA by a few instructions so that it does not wait
+  // for it). Only the last pair's stores come after the last MFMA. The stores of
+  // the launch are thereby spread over the last two and a half steps.
+  // K in whole chunks, unpaired fragment layouts.
+  constexpr bool TAILED = STAGGER != 0;
+  static_assert(!TAILED || (AM == 4 && BN == 4 && !RHS_I4 && !PAIR_A && !PAIR_B && KIND != kF32), "staggered tail");
+  // Output addressing of this wavefront's fragments, as in store_block: the byte offset of quad (j, q) from the
+  // sub-block's first column tile, whether it lies inside the matrix, and the pointer of a fragment row's line.
+  typedef typename AccType<KIND>::scalar out_scalar_t;
+  typedef out_scalar_t out_quad_t __attribute__((ext_vector_type(4)));
+  typedef typename std::conditional<NARROW, uint2, out_quad_t>::type out_stored_t;
+  constexpr int OUT_BYTES = NARROW ? 2 : 4;
+  struct OutAddressing {
+    uint8_t* wave_out;
+    uint32_t col_off[BN][4];
+    uint32_t col_inside;
+  };
+  auto out_addressing = [&]() -> OutAddressing {
+    OutAddressing o;
+    const int32_t N0 = 1 << a.log2_N0;
+    const int64_t wave_col = first_col + wave_n * (32 * BN);
+    const int64_t first_col_tile = wave_col >> a.log2_N0;
+    o.wave_out = a.out + OUT_BYTES * (first_col_tile << (a.log2_M0 + a.log2_N0));
+    o.col_inside = 0;
+#pragma unroll
+    for (int j = 0; j < BN; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int64_t col = wave_col + 4 * (lane >> 5) + 32 * j + 8 * q;
+        o.col_off[j][q] = (uint32_t)(OUT_BYTES * ((((col >> a.log2_N0) - first_col_tile) << (a.log2_M0 + a.log2_N0)) +
+                                                  (col & (N0 - 1))));
+        if (col < total_cols) o.col_inside |= 1u << (4 * j + q);
+      }
+    return o;
+  };
+  auto out_row_pointer = [&](const OutAddressing& o, int i, bool* inside) -> uint8_t* {
+    const int32_t M0 = 1 << a.log2_M0;
+    const int64_t this_row = first_row + wave_m * (32 * AM) + 32 * i + (lane & 31);
+    const int64_t row = min(this_row, total_rows - 1);
+    *inside = this_row < total_rows;
+    return o.wave_out + OUT_BYTES * ((row >> a.log2_M0) * a.out_stride0 + ((row & (M0 - 1)) << a.log2_N0));
+  };
+  constexpr int OUT_EBITS = KIND == kF16 ? 5 : 8;
+  auto out_to_float = [](out_stored_t w) -> out_quad_t {
+    if constexpr (NARROW) {
+      return out_quad_t{widen16<OUT_EBITS>((uint16_t)w.x), widen16<OUT_EBITS>((uint16_t)(w.x >> 16)),
+                        widen16<OUT_EBITS>((uint16_t)w.y), widen16<OUT_EBITS>((uint16_t)(w.y >> 16))};
+    } else {
+      return w;
+    }
+  };
+  auto out_to_stored = [](out_quad_t v) -> out_stored_t {
+    if constexpr (NARROW) {
+      return make_uint2((uint32_t)narrow16<OUT_EBITS>(v.x) | ((uint32_t)narrow16<OUT_EBITS>(v.y) << 16),
+                        (uint32_t)narrow16<OUT_EBITS>(v.z) | ((uint32_t)narrow16<OUT_EBITS>(v.w) << 16));
+    } else {
+      return v;
+    }
+  };
+
+  auto tail = [&](auto cur_a, auto cur_b) {  // (generic: only instantiated where it is called)
+    constexpr int JR = AHEAD - 1;            // chunks in the ring
+    constexpr int PAIR_MFMAS = 4 * JR;       // two fragments x JR chunks x two K-steps
+    static_assert(PAIR_MFMAS >= 8, "a quad of the previous pair is stored with each MFMA");
+    const OutAddressing o = out_addressing();
+
+    // Fragment f of an operand, K-step kk, from the stage whose per-lane bases are given.
+    auto read_fragment = [&](const uint8_t* base_a, const uint8_t* base_a_kk1, const uint8_t* base_b, bool is_b, int f,
+                             int kk) -> uint4 {
+      const uint8_t* src = is_b ? base_b : base_a;
+      if constexpr (G == 16) {
+        if (is_b) return *(const uint4*)(src + (128 * f + KK16 * kk) * 16);
+        return *(const uint4*)((kk ? base_a_kk1 : base_a) + 128 * f * 16);
+      } else if constexpr (G == 1) {
+        const uint2 lo = lds_read_transposed(src + 2048 * f + 512 * kk);
+        const uint2 hi = lds_read_transposed(src + 2048 * f + 512 * kk + 128);
+        return make_uint4(lo.x, lo.y, hi.x, hi.y);
+      } else if constexpr (G == 8) {
+        const uint8_t* first = src + 1024 * (2 * f + kk);
+        const uint2 lo = *(const uint2*)first, hi = *(const uint2*)(first + 512);
+        return make_uint4(lo.x, lo.y, hi.x, hi.y);
+      } else {
+        const uint8_t* first = src + 1024 * (2 * f + kk);
+        return make_uint4(gather_dword(first, 0), gather_dword(first, 1), gather_dword(first, 2), gather_dword(first, 3));
+      }
+    };
+    // Per-lane bases of the ring chunks' stages.
+    const uint8_t* base_a[JR];
+    const uint8_t* base_a_kk1[JR];
+    const uint8_t* base_b[JR];
+    {
+      uint32_t stage_off = read_stage_off;
+#pragma unroll
+      for (int c = 0; c < JR; ++c) {
+        base_a[c] = ring_bytes + stage_off + frag_a_off + pair_a_lane;
+        base_a_kk1[c] = base_a[c] + lhs_kk1_step;
+        base_b[c] = ring_bytes + stage_off + frag_b_off + pair_b_lane;
+        stage_off = stage_off + STAGE_BYTES == RING_BYTES ? 0 : stage_off + STAGE_BYTES;
+      }
+    }
+    uint4 tb[BN][JR][2], ta[2][JR][2];
+    // The reads of the register phase, in the order the first pair needs them: per chunk and K-step the first
+    // lhs row and the first two rhs fragments, then the other two rhs fragments.
+    constexpr int EARLY_READS = 2 * JR * (1 + BN);
+    auto early_read = [&](int n) {
+      const int half = n / (2 * JR * 3);  // 0: lhs row 0 and rhs 0, 1; 1: rhs 2, 3
+      if (half == 0) {
+        const int c = n / 6, kk = (n / 3) % 2, what = n % 3;
+        if (what == 0) ta[0][c][kk] = read_fragment(base_a[c], base_a_kk1[c], base_b[c], false, 0, kk);
+        else tb[what - 1][c][kk] = read_fragment(base_a[c], base_a_kk1[c], base_b[c], true, what - 1, kk);
+      } else {
+        const int m = n - 2 * JR * 3, c = m / 4, kk = (m / 2) % 2, j = 2 + m % 2;
+        tb[j][c][kk] = read_fragment(base_a[c], base_a_kk1[c], base_b[c], true, j, kk);
+      }
+    };
+
+    // Register phase: the chunk whose fragments are in `cur`, in the usual order.
+    constexpr int REG_MFMAS = 2 * AM * BN;
+    constexpr int WAIT_AT = REG_MFMAS - 20 > 4 ? 12 : 4;  // MFMAs ahead of the wait for the ring chunks' loads
+#pragma unroll
+    for (int m = 0; m < REG_MFMAS; ++m) {
+      if (m == WAIT_AT) {
+        wait_loads_but<0>();
+        __builtin_amdgcn_s_barrier();
+      }
+      if (m >= WAIT_AT) {
+        constexpr int SLOTS = REG_MFMAS - WAIT_AT;
+#pragma unroll
+        for (int n = (m - WAIT_AT) * EARLY_READS / SLOTS; n < (m - WAIT_AT + 1) * EARLY_READS / SLOTS; ++n) early_read(n);
+      }
+      const int kk = m / (AM * BN), i = (m % (AM * BN)) / BN, j = m % BN;
+      acc[i][j] = mfma<KIND>(cur_b[j][kk], cur_a[i][kk], acc[i][j]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // Fragment phase. (The accumulators are pinned where they are, here and again before each pair is stored:
+    // left alone, the compiler moves them to ordinary registers ahead of the stores, and there are not that many.)
+#pragma unroll
+    for (int i = 0; i < AM; ++i)
+#pragma unroll
+      for (int j = 0; j < BN; ++j) asm volatile("" : "+a"(acc[i][j]));
+    uint8_t* prev_row = nullptr;
+    bool prev_row_inside = false;
+    // Quad n (fragment n / 4 of the pair, quad n % 4) of pair (i, jp). An accumulating call adds what the
+    // destination held, loaded while the pair was multiplied (one quad per MFMA, each into the register the
+    // previous pair's quad of the same number has just been added from).
+    constexpr bool ACCUMULATING = STAGGER == 2;
+    out_quad_t old[2][4];
+    auto store_quad = [&](int i, int jp, int n, uint8_t* row_out, bool row_inside) {
+      const int t = n / 4, q = n % 4, j = 2 * jp + t;
+      out_quad_t v = out_quad_t{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+      if constexpr (ACCUMULATING) v += old[t][q];
+      if (row_inside && (o.col_inside >> (4 * j + q) & 1)) *(out_stored_t*)(row_out + o.col_off[j][q]) = out_to_stored(v);
+    };
+    auto load_old = [&](int jp, int n, const uint8_t* row_out, bool row_inside) {
+      const int t = n / 4, q = n % 4, j = 2 * jp + t;
+      old[t][q] = out_quad_t{0, 0, 0, 0};
+      if (row_inside && (o.col_inside >> (4 * j + q) & 1))
+        old[t][q] = out_to_float(*(const out_stored_t*)(row_out + o.col_off[j][q]));
+    };
+#pragma unroll
+    for (int i = 0; i < AM; ++i) {
+      bool row_inside;
+      uint8_t* row_out = out_row_pointer(o, i, &row_inside);
+#pragma unroll
+      for (int jp = 0; jp < BN / 2; ++jp) {
+        const int pair = i * (BN / 2) + jp;
+#pragma unroll
+        for (int m = 0; m < PAIR_MFMAS; ++m) {
+          // The previous pair's quads, from the third MFMA on (its last MFMA has left the pipe by then).
+          constexpr int STORE_FROM = PAIR_MFMAS >= 10 ? 2 : 0;
+          const int n = m - STORE_FROM;
+          if (n >= 0 && n < 8) {
+            if (pair > 0) {
+              const int pi = (pair - 1) / (BN / 2), pjp = (pair - 1) % (BN / 2);
+              if (n == 0) asm volatile("" : "+a"(acc[pi][2 * pjp]), "+a"(acc[pi][2 * pjp + 1]));
+              store_quad(pi, pjp, n, pi == i ? row_out : prev_row, pi == i ? row_inside : prev_row_inside);
+            }
+            if constexpr (ACCUMULATING) load_old(jp, n, row_out, row_inside);
+          }
+          // The next row's lhs fragments, read under this row's second pair.
+          if (jp == BN / 2 - 1 && i + 1 < AM && m < 2 * JR)
+            ta[(i + 1) & 1][m / 2][m % 2] = read_fragment(base_a[m / 2], base_a_kk1[m / 2], base_b[m / 2], false, i + 1, m % 2);
+          const int c = m / 4, kk = (m / 2) % 2, t = m % 2, j = 2 * jp + t;
+          acc[i][j] = mfma<KIND>(tb[j][c][kk], ta[i & 1][c][kk], acc[i][j]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      prev_row = row_out;
+      prev_row_inside = row_inside;
+    }
+    // The last pair's quads.
+    asm volatile("" : "+a"(acc[AM - 1][BN - 2]), "+a"(acc[AM - 1][BN - 1]));
+#pragma unroll
+    for (int n = 0; n < 8; ++n) store_quad(AM - 1, BN / 2 - 1, n, prev_row, prev_row_inside);
+  };
+
 #pragma unroll
   for (int c = 0; c < AHEAD; ++c) issue_chunk(c);
   wait_loads_but<(AHEAD - 1) * LOADS>();
@@ -1137,6 +1356,28 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
     }
   }
   int kc = 0;
+  if constexpr (TAILED) {
+    // (The host launches this variant only for K in whole chunks, at least 2 * STAGES of them.)
+    // An odd step first, so that the loop always ends with the next chunk's fragments in (pa, pb).
+    const int main_steps = chunks - AHEAD;
+    if (main_steps & 1) {
+      step(pa, pb, qa, qb);
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+        for (int i = 0; i < AM; ++i) pa[i][kk] = qa[i][kk];
+#pragma unroll
+        for (int j = 0; j < BN; ++j) pb[j][kk] = qb[j][kk];
+      }
+      kc = 1;
+    }
+    for (; kc + 1 < main_steps; kc += 2) {
+      step(pa, pb, qa, qb);
+      step(qa, qb, pa, pb);
+    }
+    tail(pa, pb);
+    return;
+  }
   for (; kc + 1 < chunks; kc += 2) {
     step(pa, pb, qa, qb);
     step(qa, qb, pa, pb);
@@ -1417,7 +1658,14 @@ hipError_t launch_direct(MfmaArgs m, hipStream_t stream) {
   constexpr int stage_pieces = 256 * AM + (RHS_I4 ? 128 : 256) * BN;
   constexpr size_t lds_bytes = (size_t)STAGES * 16 * stage_pieces;
   static_assert(lds_bytes <= 160 * 1024, "ring does not fit the LDS");
-  auto kernel = mmt4d_mfma_direct_kernel<KIND, RHS_I4, NARROW, G, AM, BN, STAGES>;
+  void (*kernel)(const MfmaArgs) = mmt4d_mfma_direct_kernel<KIND, RHS_I4, NARROW, G, AM, BN, STAGES>;
+  // The 256x256 tile with the staggered tail: K in whole chunks, enough of them.
+  if constexpr (AM == 4 && BN == 4 && !RHS_I4 && G != 2 && KIND != kF32) {
+    if (((int64_t)m.K * m.lhs_rb) % 64 == 0 && m.chunks >= 2 * STAGES) {
+      if (m.accumulate) kernel = mmt4d_mfma_direct_kernel<KIND, RHS_I4, NARROW, G, AM, BN, STAGES, 2>;
+      else kernel = mmt4d_mfma_direct_kernel<KIND, RHS_I4, NARROW, G, AM, BN, STAGES, 1>;
+    }
+  }
   // Above 64 KiB of dynamic LDS the limit has to be raised (per device, so it
   // is simply done on every launch: it only sets a field).
   if (lds_bytes > 65536) {
@@ -1537,7 +1785,10 @@ hipError_t launch_variant(const MfmaArgs& m, hipStream_t stream, const char** na
   switch (choose_tile<RHS_I4>(m, direct, &tile)) {
     case 0:
       *name = "mmt4d_mfma_256x256";
-      if (direct) return launch_direct<KIND, RHS_I4, NARROW, G, 4, 4, 4>(m, stream);
+#ifndef UK_STAGES_256
+#define UK_STAGES_256 4
+#endif
+      if (direct) return launch_direct<KIND, RHS_I4, NARROW, G, 4, 4, UK_STAGES_256>(m, stream);
       return launch_staged<KIND, RHS_I4, NARROW, G, 4, 4, 1>(m, stream);
     case 1:
       *name = "mmt4d_mfma_256x128";
