@@ -125,6 +125,53 @@ def _sustained_ceiling(torch, abi, synth):
                     "no prologue, no store"}
 
 
+def _in_kernel_timeline(torch, synth):
+    """Where the time of one headline launch goes, from readings of the 100 MHz counter inside the kernel (the
+    benchmark's probe: the library's kernel source compiled once more with its timeline readings on). Medians over
+    the 256 workgroups, in microseconds, for the kernel as launched (staggered tail: the last three chunks are
+    multiplied fragment by fragment and stored as they finish) and for the variant that stores everything
+    after the loop."""
+    import numpy as np
+    from iree_amd import library
+    probe = library.load_bench_probe()
+    lhs = torch.from_numpy(synth.uniform_int8(0, 0, 4096 * 4096)).cuda()
+    rhs = torch.from_numpy(synth.uniform_int8(0, 1, 4096 * 4096)).cuda()
+    out = torch.empty(4096 * 4096, dtype=torch.int32, device="cuda")
+    res = {}
+    for name, staggered in (("staggered_tail", 1), ("all_stores_after_the_loop", 0)):
+        readings = (C.c_double * (256 * 5))()
+        tiles = C.c_int()
+        rc = probe.uk_bench_probe_mmt4d_timeline(lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), 512, 512, 1024, 8, 8, 4,
+                                                 staggered, 400, 10, readings, C.byref(tiles))
+        if rc != 0:
+            raise RuntimeError("timeline probe failed: HIP error %d" % rc)
+        t = np.array(readings[:5 * tiles.value]).reshape(tiles.value, 5) / 1e3
+        med = lambda x: round(float(np.median(x)), 2)
+        res[name] = {"prologue_us": med(t[:, 1] - t[:, 0]), "main_loop_us": med(t[:, 2] - t[:, 1]),
+                     "tail_until_last_mfma_us": med(t[:, 3] - t[:, 2]),
+                     "stores_after_last_mfma_until_acknowledged_us": med(t[:, 4] - t[:, 3]),
+                     "first_start_to_last_end_us": round(float(t[:, 4].max()), 2),
+                     "workgroup_starts_spread_us": round(float(t[:, 0].max()), 2)}
+    # The two variants timed from outside, alternating, 4 x 50 launches each.
+    stream = torch.cuda.current_stream().cuda_stream
+    totals = {1: 0.0, 0: 0.0}
+    for _ in range(4):
+        for staggered in (1, 0):
+            def launch():
+                rc = probe.uk_bench_probe_mmt4d_launch(lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), 512, 512, 1024,
+                                                       8, 8, 4, staggered, stream)
+                if rc != 0:
+                    raise RuntimeError("timeline probe failed: HIP error %d" % rc)
+            ms, _ = _time_launches(torch, launch, 50, 5)
+            totals[staggered] += ms / 4
+    res["staggered_tail"]["launch_us_back_to_back"] = round(totals[1] * 1e3, 2)
+    res["all_stores_after_the_loop"]["launch_us_back_to_back"] = round(totals[0] * 1e3, 2)
+    res["what"] = ("s8s8s32 4096^3 tiles 8x8x4; 100 MHz counter read by wavefront 0 of each of the 256 workgroups, last of "
+                   "five back-to-back launches, averaged over ten such groups after 400 warm-up launches; medians over the "
+                   "workgroups. launch_us_back_to_back: the same two kernels timed by events, alternating, 4 x 50 launches")
+    return res
+
+
 def _e2e_chain(torch, lib, abi, synth, steps, warmup):
     """The chain the reference's matmul benchmark runs (tools/e2e_matmul_benchmark.c:173-186):
     pack lhs, pack rhs (given as [K, N], both transposes), mmt4d, unpack, on row-major int8
@@ -292,6 +339,7 @@ def _also(torch, lib, abi, synth, steps, warmup):
     except Exception as exc:
         res["vendor_library_f16_gemm_4096_for_comparison"] = {"unavailable": str(exc)[:200]}
     res["e2e_pack_mmt4d_unpack_s8s8s32_4096"] = _e2e_chain(torch, lib, abi, synth, steps, warmup)
+    res["mmt4d_s8s8s32_4096_in_kernel_timeline"] = _in_kernel_timeline(torch, synth)
     # What the matrix pipe sustains on this device, measured by the
     # benchmark's probe (a helper library of its own): the 256x256 kernel's inner-loop instruction mix with no
     # HBM traffic, no prologue and no epilogue, on all-zero bytes, on the

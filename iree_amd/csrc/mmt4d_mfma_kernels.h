@@ -571,6 +571,16 @@ __global__ __launch_bounds__(256, MIN_BLOCKS) void mmt4d_mfma_kernel(const MfmaA
 // enforced by hand with s_waitcnt vmcnt + a workgroup barrier once per chunk.
 extern __shared__ uint4 ring[];
 
+// Measuring aid, compiled in only by the benchmark's probe library (csrc/bench/probe_mmt4d_timeline.hip):
+// wavefront 0 of each of the first 256 workgroups leaves five readings of the constant-rate 100 MHz
+// counter (start, main loop begins, main loop ends, last MFMA issued, stores acknowledged).
+#ifdef UK_KERNEL_TIMELINE
+#define UK_TIMELINE(...) __VA_ARGS__
+__device__ unsigned long long uk_timeline[256 * 8];
+#else
+#define UK_TIMELINE(...)
+#endif
+
 // One wavefront-wide load of 64 x 16 bytes to LDS byte offset `lds_off`
 // (wavefront-uniform) from `base` (uniform) + per-lane byte offset `voff`.
 __device__ __forceinline__ void load_to_lds(uint32_t lds_off, uint32_t voff, const uint8_t* base) {
@@ -632,6 +642,8 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   static_assert(A_PIECES % 256 == 0 && B_PIECES % 256 == 0, "block tile too small");
   static_assert((AHEAD - 1) * LOADS <= 63, "the loads in flight must fit the 6-bit counter");
 
+  UK_TIMELINE(const unsigned long long tl_start = __builtin_amdgcn_s_memrealtime(); unsigned long long tl_loop = 0,
+              tl_loop_end = 0;)
   int tile_row, tile_col;
   if (!locate_block(a, &tile_row, &tile_col)) return;
 
@@ -1316,9 +1328,16 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
       prev_row_inside = row_inside;
     }
     // The last pair's quads.
+    UK_TIMELINE(const unsigned long long tl_last_mfma = __builtin_amdgcn_s_memrealtime();)
     asm volatile("" : "+a"(acc[AM - 1][BN - 2]), "+a"(acc[AM - 1][BN - 1]));
 #pragma unroll
     for (int n = 0; n < 8; ++n) store_quad(AM - 1, BN / 2 - 1, n, prev_row, prev_row_inside);
+    UK_TIMELINE(asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                if (lane == 0 && wave == 0 && blockIdx.x < 256) {
+                  unsigned long long* t = uk_timeline + blockIdx.x * 8;
+                  t[0] = tl_start; t[1] = tl_loop; t[2] = tl_loop_end; t[3] = tl_last_mfma;
+                  t[4] = __builtin_amdgcn_s_memrealtime();
+                })
   };
 
 #pragma unroll
@@ -1355,6 +1374,7 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
       }
     }
   }
+  UK_TIMELINE(tl_loop = __builtin_amdgcn_s_memrealtime();)
   int kc = 0;
   if constexpr (TAILED) {
     // (The host launches this variant only for K in whole chunks, at least 2 * STAGES of them.)
@@ -1375,6 +1395,7 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
       step(pa, pb, qa, qb);
       step(qa, qb, pa, pb);
     }
+    UK_TIMELINE(tl_loop_end = __builtin_amdgcn_s_memrealtime();)
     tail(pa, pb);
     return;
   }
@@ -1385,9 +1406,16 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   if (kc < chunks) step(pa, pb, qa, qb);
   // No load may still be writing LDS when the workgroup's allocation is freed.
   wait_loads_but<0>();
+  UK_TIMELINE(tl_loop_end = __builtin_amdgcn_s_memrealtime();)
 
   store_block<KIND, RHS_I4, NARROW, AM, BN, PAIR_A, PAIR_B>(a, acc, first_row + wave_m * (32 * AM),
                                                             first_col + wave_n * (32 * BN), lane);
+  UK_TIMELINE(asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+              if (lane == 0 && wave == 0 && blockIdx.x < 256) {
+                unsigned long long* t = uk_timeline + blockIdx.x * 8;
+                t[0] = tl_start; t[1] = tl_loop; t[2] = tl_loop_end; t[3] = tl_loop_end;
+                t[4] = __builtin_amdgcn_s_memrealtime();
+              })
 }
 
 // (Overloads on scalars rather than a bit cast of a vector element.)
@@ -1652,7 +1680,7 @@ void set_tile_grid(MfmaArgs* m, int block_rows, int block_cols, unsigned* grid) 
 
 // Direct-to-LDS kernel on (64*AM) x (64*BN) block tiles with a ring of STAGES stages.
 template <int KIND, bool RHS_I4, bool NARROW, int G, int AM, int BN, int STAGES>
-hipError_t launch_direct(MfmaArgs m, hipStream_t stream) {
+hipError_t launch_direct(MfmaArgs m, hipStream_t stream, bool staggered_tail = true) {
   unsigned grid;
   set_tile_grid(&m, 64 * AM, 64 * BN, &grid);
   constexpr int stage_pieces = 256 * AM + (RHS_I4 ? 128 : 256) * BN;
@@ -1661,7 +1689,7 @@ hipError_t launch_direct(MfmaArgs m, hipStream_t stream) {
   void (*kernel)(const MfmaArgs) = mmt4d_mfma_direct_kernel<KIND, RHS_I4, NARROW, G, AM, BN, STAGES>;
   // The 256x256 tile with the staggered tail: K in whole chunks, enough of them.
   if constexpr (AM == 4 && BN == 4 && !RHS_I4 && G != 2 && KIND != kF32) {
-    if (((int64_t)m.K * m.lhs_rb) % 64 == 0 && m.chunks >= 2 * STAGES) {
+    if (staggered_tail && ((int64_t)m.K * m.lhs_rb) % 64 == 0 && m.chunks >= 2 * STAGES) {
       if (m.accumulate) kernel = mmt4d_mfma_direct_kernel<KIND, RHS_I4, NARROW, G, AM, BN, STAGES, 2>;
       else kernel = mmt4d_mfma_direct_kernel<KIND, RHS_I4, NARROW, G, AM, BN, STAGES, 1>;
     }

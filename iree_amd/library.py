@@ -69,9 +69,10 @@ _bench_probe = None
 
 def load_bench_probe():
     """The benchmark's probes (csrc/bench/), a helper library of its own: what the
-    matrix pipe sustains on given operand bytes, and what the device streams to
-    and from HBM with plain read, fill and copy kernels. Not part of the
-    microkernel ABI."""
+    matrix pipe sustains on given operand bytes, what the device streams to and
+    from HBM with plain read, fill and copy kernels, and where the time of one
+    launch of the 256x256 int8 kernel goes (the kernel's own source compiled
+    with its timeline readings on). Not part of the microkernel ABI."""
     global _bench_probe
     if _bench_probe is None:
         path = os.path.join(HERE, "libuk_bench_probe.so")
@@ -84,5 +85,12 @@ def load_bench_probe():
         l.uk_bench_probe_hbm_stream.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_longlong, C.c_int, C.c_int,
                                                 C.c_int, C.c_void_p, C.c_void_p]
         l.uk_bench_probe_hbm_stream.restype = C.c_int
+        l.uk_bench_probe_mmt4d_timeline.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_longlong, C.c_longlong,
+                                                    C.c_longlong, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
+                                                    C.POINTER(C.c_double), C.POINTER(C.c_int)]
+        l.uk_bench_probe_mmt4d_timeline.restype = C.c_int
+        l.uk_bench_probe_mmt4d_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_longlong, C.c_longlong,
+                                                  C.c_longlong, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
+        l.uk_bench_probe_mmt4d_launch.restype = C.c_int
         _bench_probe = l
     return _bench_probe
