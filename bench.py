@@ -551,6 +551,16 @@ def _also(torch, lib, abi, synth, steps, warmup):
     timed_pair("pack_f32_8191x8190_transpose_both_to_512x8191x16x1", pack_rhs, (R * Cc + 512 * R * 16) * 4)
     del packed3
 
+    # Every second element of each row (in_stride1 = 2, as the reference's tests draw it,
+    # tools/pack_test.c:80-93): [8191, 4095] out of the same buffers into [512, 4095, 16, 1]. Counted are the
+    # elements read and written; the lines fetched hold twice the elements read.
+    def pack_strided(i):
+        p = pack_params(i, 0, 512, Cc // 2, 16, 1)
+        p.in_stride1, p.in_size1 = 2, Cc // 2
+        return (lib.iree_uk_pack_p, p)
+    timed_pair("pack_f32_8191x4095_element_stride_2_to_512x4095x16x1", pack_strided,
+               (R * (Cc // 2) + 512 * (Cc // 2) * 16) * 4)
+
     def unpack_params(i):
         p = abi.UnpackParams()
         p.in_buffer, p.out_buffer = packed[i].data_ptr(), back[i].data_ptr()

@@ -24,8 +24,13 @@
 // LDS image that is already in tiled order; the tiled side then is one 128-bit
 // LDS read and one 128-bit store per vector.
 //
-// Anything this file does not cover (non power-of-two tiles, inner stride on
-// the 2-D side, unaligned tiled buffers) goes to the generic kernels.
+// With an element stride on the 2-D side (in_stride1 / out_stride1 other than
+// 1, which the reference handles in its tile path through a temporary row,
+// pack.c:227) the 2-D side is accessed element by element, the stride apart;
+// the LDS image and the tiled side stay as they are.
+//
+// Anything this file does not cover (non power-of-two tiles, unaligned tiled
+// buffers) goes to the generic kernels.
 #include <mutex>
 #include <type_traits>
 #include <vector>
@@ -43,6 +48,7 @@ struct TiledArgs {
   const uint8_t* src;   // pack: 2-D buffer, unpack: tiled buffer
   uint8_t* dst;         // pack: tiled buffer, unpack: 2-D buffer
   int64_t flat_stride0;   // 2-D side row stride, elements
+  int64_t flat_stride1;   // 2-D side element stride, elements (1: rows are contiguous)
   int64_t tiled_stride0;  // tiled side outer stride, elements
   int64_t size0, size1;   // 2-D sizes
   int64_t outer0, outer1; // tile counts along 2-D dims 0 / 1
@@ -177,7 +183,9 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
   };
 
   // ---- 2-D rows -> LDS (pack), all global loads issued before the LDS stores ----
-  auto flat_load_phase = [&]() {
+  // (STRIDED: elements of a row lie flat_stride1 elements apart.)
+  auto flat_load_phase = [&](auto strided) {
+    constexpr bool STRIDED = decltype(strided)::value;
     constexpr int BATCH = FLAT_PER_THREAD < 8 ? FLAT_PER_THREAD : 8;
     for (int u0 = 0; u0 < FLAT_PER_THREAD; u0 += BATCH) {
       FlatVec regs[BATCH];
@@ -186,8 +194,8 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
         const int32_t v = tid + 256 * (u0 + u);
         const int32_t r = v >> log2_vpr, cv = v & vpr_mask;
         const int64_t row = row_base + r, col = col_base + (int64_t)cv * EPV;
-        const uint8_t* g = a.src + (row * a.flat_stride0 + col) * E;
-        if (row < a.size0 && col + EPV <= a.size1) {
+        const uint8_t* g = a.src + (row * a.flat_stride0 + (STRIDED ? col * a.flat_stride1 : col)) * E;
+        if (!STRIDED && row < a.size0 && col + EPV <= a.size1) {
           // Every byte is read once: streaming (non-temporal) accesses on both
           // sides leave the caches to the other side's partial lines.
           if constexpr (W == 16) {
@@ -202,7 +210,7 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
 #pragma unroll
           for (int i = 0; i < EPV; ++i) {
             elem_t x = (elem_t)a.padding_value;
-            if (row < a.size0 && col + i < a.size1) x = ((const elem_t*)g)[i];
+            if (row < a.size0 && col + i < a.size1) x = ((const elem_t*)g)[STRIDED ? i * a.flat_stride1 : i];
             regs[u].elem[i] = x;
           }
         }
@@ -217,7 +225,8 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
   };
 
   // ---- LDS -> 2-D rows (unpack), nothing written outside size0 x size1 ----
-  auto flat_store_phase = [&]() {
+  auto flat_store_phase = [&](auto strided) {
+    constexpr bool STRIDED = decltype(strided)::value;
     constexpr int BATCH = FLAT_PER_THREAD < 8 ? FLAT_PER_THREAD : 8;
     for (int u0 = 0; u0 < FLAT_PER_THREAD; u0 += BATCH) {
       FlatVec regs[BATCH];
@@ -231,8 +240,8 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
         const int32_t v = tid + 256 * (u0 + u);
         const int32_t r = v >> log2_vpr, cv = v & vpr_mask;
         const int64_t row = row_base + r, col = col_base + (int64_t)cv * EPV;
-        uint8_t* g = a.dst + (row * a.flat_stride0 + col) * E;
-        if (row < a.size0 && col + EPV <= a.size1) {
+        uint8_t* g = a.dst + (row * a.flat_stride0 + (STRIDED ? col * a.flat_stride1 : col)) * E;
+        if (!STRIDED && row < a.size0 && col + EPV <= a.size1) {
           // Whole vectors inside the matrix: written once, not read here.
           if constexpr (W == 16) {
             typedef int v4a1 __attribute__((ext_vector_type(4), aligned(1)));
@@ -247,7 +256,7 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
         } else if (row < a.size0) {
 #pragma unroll
           for (int i = 0; i < EPV; ++i)
-            if (col + i < a.size1) ((elem_t*)g)[i] = regs[u].elem[i];
+            if (col + i < a.size1) ((elem_t*)g)[STRIDED ? i * a.flat_stride1 : i] = regs[u].elem[i];
         }
       }
     }
@@ -297,13 +306,13 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
   };
 
   if constexpr (!UNPACK) {
-    flat_load_phase();
+    if (a.flat_stride1 == 1) flat_load_phase(std::false_type()); else flat_load_phase(std::true_type());
     __syncthreads();
     tiled_phase();
   } else {
     tiled_phase();
     __syncthreads();
-    flat_store_phase();
+    if (a.flat_stride1 == 1) flat_store_phase(std::false_type()); else flat_store_phase(std::true_type());
   }
 }
 
@@ -616,7 +625,7 @@ bool make_plan(const uint8_t* flat, const uint8_t* tiled, int64_t flat_stride0, 
                int64_t tiled_stride0, int64_t size0, int64_t size1, int64_t tsize0, int64_t tsize1,
                int64_t tsize2, int64_t tsize3, bool tr_inner, bool tr_outer, int elem_bytes,
                bool for_unpack, Plan* plan) {
-  if (flat_stride1 != 1) return false;
+  if (flat_stride1 < 1) return false;  // (0: every element of a row the same one; left to the generic kernel)
   const int l2 = log2_exact(tsize2), l3 = log2_exact(tsize3);
   if (l2 < 0 || l3 < 0) return false;
   const int64_t tile_bytes = tsize2 * tsize3 * elem_bytes;
@@ -634,6 +643,7 @@ bool make_plan(const uint8_t* flat, const uint8_t* tiled, int64_t flat_stride0, 
   a.outer0 = tr_outer ? tsize1 : tsize0;
   a.outer1 = tr_outer ? tsize0 : tsize1;
   a.flat_stride0 = flat_stride0;
+  a.flat_stride1 = flat_stride1;
   a.tiled_stride0 = tiled_stride0;
   a.size0 = size0;
   a.size1 = size1;
@@ -816,7 +826,7 @@ void choose_transposing_wide(TiledArgs* a, int elem_bytes) {
 int plan_transposing(Plan* p) {
   TiledArgs& a = p->args;
   const int E = p->elem_bytes;
-  if (!a.tr_inner || E > 2 || p->flat_vec_bytes != 16) return 0;
+  if (!a.tr_inner || E > 2 || p->flat_vec_bytes != 16 || a.flat_stride1 != 1) return 0;
   const int log2_e = E == 2 ? 1 : 0;
   const int log2_rq = 2 - log2_e, log2_ve = 4 - log2_e;
   if (a.log2_bc + log2_e < 4) return 0;
