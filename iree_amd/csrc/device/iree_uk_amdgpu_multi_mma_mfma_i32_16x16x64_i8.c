@@ -39,11 +39,21 @@
 // (the same bytes to the same place).
 //
 // The load instruction takes its workgroup-memory address from the M0
-// register, which the inline assembly below sets without the compiler knowing
-// (there is no clobber it accepts for M0): a function this is inlined into must
-// not rely on M0 keeping a value across the call. Compiled code uses M0 for
-// LDS-DMA builtins, indirect register indexing, s_sendmsg and readlane-style
-// moves; the loops here index their register arrays with constants only.
+// register. The compiler accepts no clobber for M0, and this function is
+// inlined into dispatches the compiler generates, which may keep a value of
+// their own in M0 (LDS-DMA builtins, indirect register indexing, s_sendmsg,
+// readlane-style moves): so the inline assembly below leaves M0 as it found
+// it, at the price of two scalar moves per load. The loops here index their
+// register arrays with constants only.
+//
+// Provenance: the signature, ab_tile_info_t / get_ab_tile_info (in the
+// shared-memory header), the thread-relative offset arithmetic at the top of
+// the microkernel, the loops that load and store the C registers and the
+// parameter list in the comment above are the reference's, nearly as they
+// stand in the gfx942 file named above: they are the calling convention a
+// compiler generates calls against. The K loop (ring of buffers, loads straight
+// to workgroup memory, one counter wait per step, repeated groups) is this
+// library's.
 #include "common.h"
 #include "iree_uk_amdgpu_multi_mma_mfma_i32_16x16x64_i8_shared_memory.h"
 
@@ -59,8 +69,9 @@ int32_t iree_uk_amdgpu_multi_mma_mfma_i32_16x16x64_i8_query_shared_memory_bytes(
 // 64 vectors from `base` (wavefront-uniform) + lane_byte_offset to the
 // workgroup-memory address lds_address + 16 * lane.
 static inline void load_vectors_to_lds(uint32_t lds_address, const int32x4_t *base, uint32_t lane_byte_offset) {
-  __asm__ volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                   :
+  uint32_t callers_m0;
+  __asm__ volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3\n\ts_mov_b32 m0, %0"
+                   : "=&s"(callers_m0)
                    : "s"(lds_address), "v"(lane_byte_offset), "s"(base)
                    : "memory");
 }
