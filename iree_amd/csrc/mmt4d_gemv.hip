@@ -364,6 +364,114 @@ __global__ __launch_bounds__(64 * kWaves) void mmt4d_gemv_i4_kernel(const GemvAr
   }
 }
 
+// The resident-lhs form of the int4 kernel (see mmt4d_gemv_resident_lhs_kernel): with 16 lhs rows the int8 lhs
+// operands of a step are twice the bytes of a rhs tile's nibbles, all of it through L2 again for every tile. One
+// workgroup per compute unit, wavefront w keeps the lhs operands of its K share (two 16-byte pieces per lane
+// and step) in LDS and streams the unit's half tiles past them. Needs steps == kWaves * UNROLL.
+template <int kWaves, int UNROLL, int MAX_TILES>
+__global__ __launch_bounds__(64 * kWaves) void mmt4d_gemv_i4_resident_lhs_kernel(const GemvArgs a) {
+  extern __shared__ uint4 gemv_lds[];  // [kWaves][UNROLL][2][64] lhs operands; then [MAX_TILES][kWaves][64] partial sums
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int row = lane & 15, g = lane >> 4;
+  const int32_t M0 = 1 << a.log2_M0;
+  const int32_t lhs_rows = a.M << a.log2_M0;  // <= 16
+  const int32_t rhs_rb = a.rb >> 1, log2_rhs_rb = a.log2_rb - 1;
+  const int64_t lhs_kstep = (int64_t)a.rb << a.log2_M0;
+  const int64_t lhs_step_bytes = (int64_t)128 << a.log2_M0;
+
+  const int64_t halves = 2 * (int64_t)a.N;
+  const int64_t h0 = (int64_t)blockIdx.x * halves / gridDim.x, h1 = ((int64_t)blockIdx.x + 1) * halves / gridDim.x;
+  if (h1 <= h0) return;
+  const int64_t t0 = h0 >> 1, t1 = (h1 - 1) >> 1;
+  const int tiles = (int)(t1 - t0 + 1);  // <= MAX_TILES (checked on the host)
+  const bool skip_low_half_of_first = h0 & 1, skip_high_half_of_last = h1 & 1;
+
+  const bool lhs_valid = row < lhs_rows;
+  const int32_t first_step = wave * UNROLL;  // this wavefront's share of K
+  const uint8_t* lhs_lane = a.lhs + (int64_t)(row >> a.log2_M0) * a.lhs_stride_bytes +
+                            (int64_t)(row & (M0 - 1)) * a.rb + ((32 * g) >> a.log2_rb) * lhs_kstep +
+                            ((32 * g) & (a.rb - 1)) + first_step * lhs_step_bytes;
+  const uint8_t* rhs_lane = a.rhs + t0 * a.rhs_stride_bytes + (int64_t)row * rhs_rb +
+                            ((16 * g) >> log2_rhs_rb) * ((int64_t)rhs_rb * 16) + ((16 * g) & (rhs_rb - 1)) +
+                            (int64_t)first_step * 1024;
+
+  auto tile_rows_loaded = [&](int u) -> bool {
+    if (u == 0 && skip_low_half_of_first && row < 8) return false;
+    if (u == tiles - 1 && skip_high_half_of_last && row >= 8) return false;
+    return true;
+  };
+  // Loads of up to DEPTH - 1 tiles in flight ahead of the one being multiplied (8 KiB per wavefront and tile).
+  constexpr int DEPTH = 4;
+  uint4 r[DEPTH][UNROLL];
+  auto fetch = [&](int u, uint4* dst) {
+    const uint8_t* p = rhs_lane + (int64_t)u * a.rhs_stride_bytes;
+    const bool loaded = tile_rows_loaded(u);
+#pragma unroll
+    for (int s = 0; s < UNROLL; ++s) {
+      dst[s] = make_uint4(0, 0, 0, 0);
+      if (loaded) dst[s] = __builtin_bit_cast(uint4, __builtin_nontemporal_load((const v4i32*)(p + (int64_t)s * 1024)));
+    }
+  };
+#pragma unroll
+  for (int u = 0; u < DEPTH - 1; ++u)
+    if (u < tiles) fetch(u, r[u]);
+  uint4* own_lhs = gemv_lds + (wave * UNROLL) * 128 + lane;
+  {
+    uint4 l0[UNROLL], l1[UNROLL];
+#pragma unroll
+    for (int s = 0; s < UNROLL; ++s) {
+      l0[s] = l1[s] = make_uint4(0, 0, 0, 0);
+      if (lhs_valid) {
+        l0[s] = *(const uint4*)(lhs_lane + s * lhs_step_bytes);
+        l1[s] = *(const uint4*)(lhs_lane + s * lhs_step_bytes + 16);
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < UNROLL; ++s) {
+      own_lhs[s * 128] = l0[s];
+      own_lhs[s * 128 + 64] = l1[s];
+    }
+  }
+
+  v4i32 acc[MAX_TILES];
+#pragma unroll
+  for (int u = 0; u < MAX_TILES; ++u) acc[u] = v4i32{0, 0, 0, 0};
+#pragma unroll
+  for (int u = 0; u < MAX_TILES; ++u) {
+    if (u < tiles) {
+      if (u + DEPTH - 1 < tiles) fetch(u + DEPTH - 1, r[(u + DEPTH - 1) % DEPTH]);
+#pragma unroll
+      for (int s = 0; s < UNROLL; ++s) {
+        const uint4 w = r[u % DEPTH][s];
+        acc[u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i32, widen_i4_times16(w.x, w.y)),
+                                                       __builtin_bit_cast(v4i32, own_lhs[s * 128]), acc[u], 0, 0, 0);
+        acc[u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i32, widen_i4_times16(w.z, w.w)),
+                                                       __builtin_bit_cast(v4i32, own_lhs[s * 128 + 64]), acc[u], 0, 0, 0);
+      }
+    }
+  }
+
+  __syncthreads();  // the lhs slices are no longer read: their memory takes the partial sums
+  v4i32* partial = (v4i32*)gemv_lds;
+#pragma unroll
+  for (int u = 0; u < MAX_TILES; ++u)
+    if (u < tiles) partial[(u * kWaves + wave) * 64 + lane] = acc[u];
+  __syncthreads();
+  for (int u = wave; u < tiles; u += kWaves) {
+    if (!lhs_valid) continue;
+    if (u == 0 && skip_low_half_of_first && g < 2) continue;
+    if (u == tiles - 1 && skip_high_half_of_last && g >= 2) continue;
+    v4i32 v = partial[(u * kWaves) * 64 + lane];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) v += partial[(u * kWaves + w) * 64 + lane];
+    v = v4i32{v.x >> 4, v.y >> 4, v.z >> 4, v.w >> 4};
+    v4i32* dst = (v4i32*)(a.out + 4 * ((int64_t)(row >> a.log2_M0) * a.out_stride0 + (t0 + u) * ((int64_t)M0 * 16) +
+                                       (int64_t)(row & (M0 - 1)) * 16 + 4 * g));
+    if (a.accumulate) v += *dst;
+    *dst = v;
+  }
+}
+
 int log2_exact(int64_t v) {
   if (v <= 0 || (v & (v - 1))) return -1;
   int l = 0;
@@ -472,6 +580,23 @@ hipError_t launch_gemv(const Mmt4dArgs& a, hipStream_t stream, const char** name
   if (!make_args(a, false, &kind, &g)) return hipErrorInvalidValue;
   *name = "mmt4d_gemv";
   if (kind == kI8I4) {
+    // More than 4 lhs rows and a tile or more per compute unit: the resident-lhs kernel, where its instantiations
+    // fit the number of steps (each of 128 values of K; the lhs of 64 steps fills 128 KiB of LDS).
+    const int units = compute_units();
+    constexpr int MAX_TILES = 8;
+    if ((g.M << g.log2_M0) > 4 && units > 0 && g.N >= units && (2 * (int64_t)g.N + units - 1) / units / 2 + 1 <= MAX_TILES &&
+        (g.steps == 64 || g.steps == 32)) {
+      const int lds_bytes = 128 * 1024;  // the lhs operands of 64 steps; the partial sums need less
+      // (16 wavefronts x 4 steps with three tiles' loads in flight: 0.65 of the HBM peak at 16 x 28672 x 8192 against
+      // 0.62 for the kernel below; 8 wavefronts x 8 steps 0.63, deeper prefetch slower.)
+      void (*kernel)(const GemvArgs) = g.steps == 64 ? mmt4d_gemv_i4_resident_lhs_kernel<16, 4, MAX_TILES>
+                                                     : mmt4d_gemv_i4_resident_lhs_kernel<8, 4, MAX_TILES>;
+      const hipError_t attr = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+      if (attr != hipSuccess) return attr;
+      *name = "mmt4d_gemv_resident_lhs";
+      hipLaunchKernelGGL(kernel, dim3(units), dim3(g.steps == 64 ? 1024 : 512), lds_bytes, stream, g);
+      return hipGetLastError();
+    }
     // More than 4 lhs rows: two rhs tiles per workgroup (measured on 16 rows x
     // 65536 x 8192: 4.5 TB/s with one, 5.9 with two, 4.9 with four).
     if ((g.M << g.log2_M0) > 4) {
