@@ -34,7 +34,7 @@ PEAK_HBM_GBS = 8000.0       # HBM3E
 # WRITE_SIZE on this part). The algorithmic minimum is 32 MiB read + 64 MiB
 # written = 100.7 MB; reads above it are lhs/rhs panels fetched by more than
 # one of the 8 L2s. profiles/ holds the counter summaries.
-HEADLINE_TRAFFIC_BYTES = 165_145_395   # 47,869 KiB x 2.00 fetched + 65,536 KiB written
+HEADLINE_TRAFFIC_BYTES = 167_835_648   # 49,175.5 KiB x 2.00 fetched + 65,551 KiB written
 
 
 def _mmt4d_params(abi, lhs, rhs, out, M, N, K, M0, N0, K0, flags):

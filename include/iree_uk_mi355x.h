@@ -172,7 +172,16 @@ typedef struct iree_uk_query_tile_sizes_2d_out_params_t {
  * Replaces: mmt4d.h:14-21 (flat form), mmt4d_internal.h:35 (struct form),
  * implemented by mmt4d.c:115-177. `cpu_data` is accepted and ignored (may be
  * NULL). IREE_UK_FLAG_MMT4D_ALLOW_GENERIC_FALLBACK_TILE_FUNCTION is accepted;
- * tile shapes without an MFMA kernel always run on the generic GPU kernel. */
+ * tile shapes without an MFMA kernel always run on the generic GPU kernel.
+ * Strides (the reference checks none, mmt4d.c:12-48): lhs_stride0 and
+ * rhs_stride0 may be anything non-negative, 0 and values shorter than a panel
+ * included (panels that coincide or overlap are only read). Deviations, both
+ * reported through the failure handler with the output left untouched: output
+ * rows that overlap (M > 1 and out_stride0 < N * M0 * N0; they are written
+ * concurrently here) and negative strides where there is more than one row.
+ * Tiles one row tall (M0 = 1) make a row-major [M, K] matrix the lhs and a
+ * row-major [M, N * N0] matrix the result as they stand: no pack of the lhs
+ * and no unpack are needed then. */
 void iree_uk_mmt4d(const void* lhs_buffer, iree_uk_index_t lhs_offset,
                    iree_uk_index_t lhs_stride0, const void* rhs_buffer,
                    iree_uk_index_t rhs_offset, iree_uk_index_t rhs_stride0,
