@@ -148,16 +148,18 @@ constexpr int kBlockBytes = 16384;  // bytes of the 2-D matrix per workgroup
 // workgroups. Row r of block b then covers columns [b * BC + s(r), (b + 1) * BC
 // + s(r)), s(r) < 128 / E being the distance from the block's first column to
 // the row's next line boundary; the first block of a row starts at column 0
-// and the last one ends with the row. A block therefore reads up to ext_cols
-// columns of the tiles that follow its own, and leaves the first s(r) columns
-// of its own tiles to the block before it; a tiled-side vector none of whose
-// elements falls into the block's windows is not loaded. In LDS, row r holds
-// its window from byte 128 on (the first block's columns below s(r) sit in
-// front of that), so the shift is paid in the element-wise LDS writes and the
-// 2-D side reads whole aligned vectors.
+// and the last one ends with the row. A block therefore also reads the
+// ext_cols columns of the tiles that follow its own. The LDS image is that of
+// the block and those columns, unmoved; the 2-D side reads row r's vectors
+// s(r) elements in (16-byte reads at element alignment). Measured on f32
+// [512, 8190, 16, 1] -> [8191, 8190]: 5.60 -> 5.88 TB/s; with the stores moved
+// but the extra columns not read (wrong results) 6.08: the 1/8 more lines
+// requested on the tiled side cost what is left, whether or not the loads are
+// masked down to the rows that are used, and although the lines shared by two
+// blocks come from HBM only once.
 template <int E, int W, int PL_BYTES, bool UNPACK, bool LINE_ALIGNED = false>
 __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
-  static_assert(!LINE_ALIGNED || (UNPACK && PL_BYTES == E && W == 16), "line-aligned unpack writes LDS element by element");
+  static_assert(!LINE_ALIGNED || (UNPACK && W == 16), "line-aligned windows are for unpack");
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   typedef typename std::conditional<E == 1, uint8_t,
           typename std::conditional<E == 2, uint16_t, uint32_t>::type>::type elem_t;
@@ -323,7 +325,6 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
   };
 
   if constexpr (LINE_ALIGNED) {
-    constexpr int HEAD = 128 / E;  // columns of LDS in front of a row's window
     constexpr int MAX_TILED = TILED_PER_THREAD + 4;
     const int32_t bc = 1 << a.log2_bc;
     const int32_t log2_tile = a.log2_t0 + a.log2_t1;
@@ -332,57 +333,59 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
     const uint32_t row_bytes = (uint32_t)((uint64_t)a.flat_stride0 * E) & 127u;
     const uint32_t to_line0 = (uint32_t)(0 - (uintptr_t)(a.dst + (row_base * a.flat_stride0 + col_base) * E)) & 127u;
     auto shift_of = [&](int32_t r) -> int32_t { return (int32_t)((to_line0 - (uint32_t)r * row_bytes) & 127u) / E; };
+    // The tiled side: the block's own tiles and the ext_cols columns of tiles
+    // after them, whole (which rows of those columns fall into this block's
+    // windows is not looked at: a partly masked load touches the same lines,
+    // and working it out ahead of the loads costs more than it saves). Nothing
+    // of the window arithmetic comes before the loads: a workgroup lives for a
+    // few microseconds, and what it computes first is time with nothing in
+    // flight. The columns around a block's edge are read by two blocks: those
+    // loads leave their lines in the cache for the other one, the rest stream.
     // A thread's vectors are 1024 elements apart, a whole number of tiles (the
-    // host sees to that): all of them are the same VE elements of their tiles.
-    // Per element: its column within the tile less the row's shift, and the LDS
-    // offset it would have in the block's first tile.
+    // host sees to that): all of them are the same pieces of their tiles.
+    typedef int v4 __attribute__((ext_vector_type(4)));
     const int32_t e0 = tid * VE, w0 = e0 & ((1 << log2_tile) - 1);
-    int32_t moved_col[VE], lds_base[VE];
-#pragma unroll
-    for (int q = 0; q < VE; ++q) {
-      const int32_t w = w0 + q, u2 = w >> a.log2_s3, u3 = w & ((1 << a.log2_s3) - 1);
-      const int32_t row = a.tr_inner ? u3 : u2;
-      moved_col[q] = (a.tr_inner ? u2 : u3) - shift_of(row);
-      lds_base[q] = row * a.pitch_bytes + (moved_col[q] + HEAD) * E;
-    }
-    // Element q of the thread's vector in tile o1l belongs to this block's windows?
-    auto stored_here = [&](int32_t o1l, int q) -> bool {
-      const int32_t c = (o1l << a.log2_t1) + moved_col[q];
-      return c < bc && (c >= 0 || first_block);
-    };
+    const uint8_t* const tile_row = a.src + (tile0_base * a.tiled_stride0 + w0) * E;
     const int32_t total_vecs = ((bc + a.ext_cols) << a.log2_br) / VE;
     TiledVec regs[MAX_TILED];
     bool wanted[MAX_TILED];
 #pragma unroll
     for (int u = 0; u < MAX_TILED; ++u) {
-      const int32_t vec = tid + 256 * u, o1l = (vec * VE) >> log2_tile;
-      wanted[u] = false;
-      if (vec < total_vecs && tile0_base < a.outer0 && tile1_base + o1l < a.outer1) {
-#pragma unroll
-        for (int q = 0; q < VE; ++q) wanted[u] = wanted[u] || stored_here(o1l, q);
-      }
+      const int32_t vec = tid + 256 * u, o1l = (vec * VE) >> log2_tile, col0 = o1l << a.log2_t1;
+      wanted[u] = vec < total_vecs && tile1_base + o1l < a.outer1;
       if (wanted[u]) {
-        typedef int v4 __attribute__((ext_vector_type(4)));
-        const int64_t global_elem = tile0_base * a.tiled_stride0 + ((tile1_base + o1l) << log2_tile) + w0;
-        regs[u].vec = __builtin_bit_cast(uint4, __builtin_nontemporal_load((const v4*)(a.src + global_elem * E)));
+        const uint8_t* g = tile_row + (((tile1_base + o1l) << log2_tile) * E);
+        if (col0 < 128 / E || col0 >= bc)
+          regs[u].vec = *(const uint4*)g;
+        else
+          regs[u].vec = __builtin_bit_cast(uint4, __builtin_nontemporal_load((const v4*)g));
       }
+    }
+    int32_t lds_base[PIECES];
+#pragma unroll
+    for (int q = 0; q < PIECES; ++q) {
+      const int32_t w = w0 + q * PL, u2 = w >> a.log2_s3, u3 = w & ((1 << a.log2_s3) - 1);
+      lds_base[q] = (a.tr_inner ? u3 : u2) * a.pitch_bytes + (a.tr_inner ? u2 : u3) * E;
     }
 #pragma unroll
     for (int u = 0; u < MAX_TILED; ++u) {
       if (!wanted[u]) continue;
       const int32_t o1l = ((tid + 256 * u) * VE) >> log2_tile;
 #pragma unroll
-      for (int q = 0; q < VE; ++q)
-        if (stored_here(o1l, q)) *(piece_t*)(lds + lds_base[q] + ((o1l << a.log2_t1) * E)) = regs[u].piece[q];
+      for (int q = 0; q < PIECES; ++q) *(piece_t*)(lds + lds_base[q] + ((o1l << a.log2_t1) * E)) = regs[u].piece[q];
     }
     __syncthreads();
     // Whole lines: vector cv of row r starts s(r) + cv * EPV columns into the block.
     {
+      struct __attribute__((packed, aligned(E))) ShiftedVec {
+        uint32_t x, y, z, w;
+      };
       FlatVec out[FLAT_PER_THREAD];
 #pragma unroll
       for (int u = 0; u < FLAT_PER_THREAD; ++u) {
-        const int32_t v = tid + 256 * u;
-        out[u].vec = *(const flat_vec_t*)(lds + (v >> log2_vpr) * a.pitch_bytes + HEAD * E + (v & vpr_mask) * W);
+        const int32_t v = tid + 256 * u, r = v >> log2_vpr;
+        const ShiftedVec t = *(const ShiftedVec*)(lds + r * a.pitch_bytes + shift_of(r) * E + (v & vpr_mask) * W);
+        out[u].vec = Dwords4{t.x, t.y, t.z, t.w};
       }
 #pragma unroll
       for (int u = 0; u < FLAT_PER_THREAD; ++u) {
@@ -402,12 +405,12 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
     }
     // A row's first columns, up to its first line boundary.
     if (first_block) {
+      constexpr int HEAD = 128 / E;
       for (int32_t i = tid; i < (HEAD << a.log2_br); i += 256) {
         const int32_t r = i / HEAD, c = i % HEAD;
         const int64_t row = row_base + r;
-        const int32_t shift = shift_of(r);
-        if (c < shift && row < a.size0 && c < a.size1)
-          ((elem_t*)(a.dst + row * a.flat_stride0 * E))[c] = *(const elem_t*)(lds + r * a.pitch_bytes + (c - shift + HEAD) * E);
+        if (c < shift_of(r) && row < a.size0 && c < a.size1)
+          ((elem_t*)(a.dst + row * a.flat_stride0 * E))[c] = *(const elem_t*)(lds + r * a.pitch_bytes + c * E);
       }
     }
   } else if constexpr (!UNPACK) {
@@ -693,10 +696,9 @@ void host_row_col(const TiledArgs& a, int32_t e, int32_t* row, int32_t* col) {
 
 // LDS row pitch: the block width plus the padding (in 16-byte steps) that
 // spreads one wavefront's tiled-side accesses over the most of the 64 banks.
-// (line_row_bytes >= 0: the line-aligned unpack, where row r's columns are
-// moved left by its distance to the next line and 128 bytes lie in front.)
-int choose_pitch(const TiledArgs& a, int elem_bytes, int piece_bytes, int line_row_bytes = -1) {
-  const int row_bytes = (1 << a.log2_bc) * elem_bytes + (line_row_bytes >= 0 ? 128 : 0);
+// (extra_cols: columns of the following tiles that the image holds as well.)
+int choose_pitch(const TiledArgs& a, int elem_bytes, int piece_bytes, int extra_cols = 0) {
+  const int row_bytes = ((1 << a.log2_bc) + extra_cols) * elem_bytes;
   const int ve = 16 / elem_bytes;
   int best_pitch = row_bytes, best_cost = 1 << 30;
   for (int pad = 0; pad <= 256; pad += 16) {
@@ -705,8 +707,7 @@ int choose_pitch(const TiledArgs& a, int elem_bytes, int piece_bytes, int line_r
     for (int lane = 0; lane < 64; ++lane) {
       int32_t row, col;
       host_row_col(a, lane * ve, &row, &col);
-      int addr = row * pitch + col * elem_bytes;
-      if (line_row_bytes >= 0) addr += 128 - (int)((0u - (unsigned)(row * line_row_bytes)) & 127u);
+      const int addr = row * pitch + col * elem_bytes;
       const int words = piece_bytes < 4 ? 1 : piece_bytes / 4;
       for (int w = 0; w < words; ++w) hits[((addr / 4) + w) & 63]++;
     }
@@ -810,12 +811,8 @@ bool make_plan(const uint8_t* flat, const uint8_t* tiled, int64_t flat_stride0, 
   plan->line_aligned = for_unpack && E == 4 && !tr_outer && flat_stride1 == 1 && size1 > bc && T0 * T1 <= 1024 &&
                        ((uintptr_t)flat % 128 != 0 || (size0 > 1 && (flat_stride0 * E) % 128 != 0));
   a.ext_cols = 0;
-  if (plan->line_aligned) {
-    piece = E;
-    plan->piece_bytes = piece;
-    a.ext_cols = (int32_t)(T1 > 128 / E ? T1 : 128 / E);
-  }
-  a.pitch_bytes = choose_pitch(a, E, piece, plan->line_aligned ? (int)((flat_stride0 * E) & 127) : -1);
+  if (plan->line_aligned) a.ext_cols = (int32_t)(T1 > 128 / E ? T1 : 128 / E);
+  a.pitch_bytes = choose_pitch(a, E, piece, a.ext_cols);
   a.blocks1 = (int32_t)((size1 + bc - 1) / bc);
   // Blocks must cover every tile of the tiled side, not only the 2-D extent
   // (pack writes whole tiles of padding beyond it).
@@ -1129,7 +1126,14 @@ hipError_t launch_unpack(const UnpackArgs& original, hipStream_t stream, const c
   plan.args.padding_value = 0;
   *name = "unpack_tiled";
   if (plan.line_aligned) {
-    hipLaunchKernelGGL((tiled_kernel<4, 16, 4, true, true>), dim3(plan.grid), dim3(256), plan.lds_bytes, stream, plan.args);
+    const dim3 grid(plan.grid), block(256);
+    if (plan.piece_bytes == 16) {
+      hipLaunchKernelGGL((tiled_kernel<4, 16, 16, true, true>), grid, block, plan.lds_bytes, stream, plan.args);
+    } else if (plan.piece_bytes == 8) {
+      hipLaunchKernelGGL((tiled_kernel<4, 16, 8, true, true>), grid, block, plan.lds_bytes, stream, plan.args);
+    } else {
+      hipLaunchKernelGGL((tiled_kernel<4, 16, 4, true, true>), grid, block, plan.lds_bytes, stream, plan.args);
+    }
     return hipGetLastError();
   }
   return launch_plan<true>(plan, stream);
