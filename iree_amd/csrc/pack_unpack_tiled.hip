@@ -66,6 +66,9 @@ struct TiledArgs {
   int32_t log2_lpr, log2_period, pad_bytes;
   int32_t band;  // rows of blocks that are walked together (block_of)
   int32_t ext_cols;  // line-aligned unpack only: columns a block reads beyond its own
+  // linear_block_of: consecutive blocks that one XCD takes, workgroups per XCD
+  // that are dealt out that way, and blocks per XCD of the rest.
+  int32_t group, grouped_slots, rest_per_xcd;
 };
 
 // Coordinates of an element of the tiled side within a block.
@@ -129,6 +132,31 @@ __device__ __forceinline__ void block_of(const TiledArgs& a, int32_t linear, int
   *block1 = i / rows_here;
 }
 
+// Workgroup id -> block number. Consecutive workgroup ids land on different
+// XCDs (separate L2s): workgroup 8 s + x runs on XCD x. Blocks are dealt to
+// the XCDs in groups of a.group consecutive numbers: within a group,
+// neighbours along a row share the cache lines at their common edge (rows
+// need not be aligned to lines) and meet in one L2; across groups, the eight
+// XCDs work side by side on one compact stretch of both buffers instead of
+// on eight stretches an eighth of the matrix apart. Measured on f32
+// [8191, 8190] with 16x1 tiles (32 blocks per row), group 1 / 16..128 / an
+// eighth of all blocks: pack 5.77 / 6.01-6.04 / 5.92 TB/s, unpack 5.99 /
+// 6.08-6.10 / 5.90, the copy-like pack into [8191, 512, 1, 16] 5.97 / 6.10-6.15
+// / 5.68; walking bands of rows (block_of), one band's blocks per group:
+// pack with both transposes 5.73 against 5.31-5.39 (groups of 16..256) and
+// 5.54 (an eighth of all blocks).
+// What does not fill eight whole groups any more is split into eight equal
+// stretches, so that no XCD is left with a group more than the others.
+__device__ __forceinline__ int32_t linear_block_of(const TiledArgs& a) {
+  const uint32_t xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, group = (uint32_t)a.group;
+  if (slot < (uint32_t)a.grouped_slots) {
+    const uint32_t g = slot / group;
+    return (int32_t)((g * 8 + xcd) * group + (slot - g * group));
+  }
+  const uint32_t r = slot - (uint32_t)a.grouped_slots;
+  return (int32_t)((uint32_t)a.grouped_slots * 8 + xcd * (uint32_t)a.rest_per_xcd + r);
+}
+
 // 16 bytes without an alignment requirement: the hardware's multi-dword
 // global accesses have none, the C++ type system would.
 struct __attribute__((packed, aligned(1))) Dwords4 {
@@ -182,12 +210,7 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
   constexpr int LOG2_W = W == 16 ? 4 : W == 8 ? 3 : W == 4 ? 2 : W == 2 ? 1 : 0;
 
   const int tid = threadIdx.x;
-  // Consecutive workgroup ids land on different XCDs (separate L2s). Regroup
-  // them so that one XCD owns a contiguous range of blocks: neighbours along a
-  // row share the cache lines at their common edge (rows need not be aligned
-  // to lines), and those then meet in one L2 instead of two.
-  const int32_t per_xcd = (a.total_blocks + 7) >> 3;
-  const int32_t linear = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int32_t linear = linear_block_of(a);
   if (linear >= a.total_blocks) return;
   int64_t block0, block1;
   block_of(a, linear, &block0, &block1);
@@ -473,8 +496,7 @@ __global__ __launch_bounds__(256) void pack_transposing_wide_kernel(const TiledA
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int lane_row = lane >> 4, cg = lane & 15;
-  const int32_t per_xcd = (a.total_blocks + 7) >> 3;
-  const int32_t linear = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int32_t linear = linear_block_of(a);
   if (linear >= a.total_blocks) return;
   int64_t block0, block1;
   block_of(a, linear, &block0, &block1);
@@ -581,8 +603,7 @@ __global__ __launch_bounds__(256) void pack_transposing_kernel(const TiledArgs a
   constexpr int TILED_PER_THREAD = kBlockBytes / 16 / 256;
 
   const int tid = threadIdx.x;
-  const int32_t per_xcd = (a.total_blocks + 7) >> 3;
-  const int32_t linear = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int32_t linear = linear_block_of(a);
   if (linear >= a.total_blocks) return;
   int64_t block0, block1;
   block_of(a, linear, &block0, &block1);
@@ -821,10 +842,19 @@ bool make_plan(const uint8_t* flat, const uint8_t* tiled, int64_t flat_stride0, 
   a.blocks1 = (int32_t)((cols_needed + bc - 1) / bc);
   if (blocks0 * a.blocks1 >= (1ll << 31)) return false;
   a.total_blocks = (int32_t)(blocks0 * a.blocks1);
-  plan->grid = (unsigned)(((a.total_blocks + 7) / 8) * 8);
   // Bytes of one contiguous run on the tiled side when runs are short.
   const int64_t run_bytes = (br / T0) * T0 * T1 * E;
   a.band = !tr_outer ? 1 : (run_bytes <= 128 ? 32 : 16);
+  // Groups of blocks per XCD (linear_block_of): 64 blocks, or one band's.
+  {
+    const int64_t group = a.band > 1 ? (int64_t)a.band * a.blocks1 : 64;
+    const int64_t grouped_slots = a.total_blocks / (8 * group) * group;
+    const int64_t rest = a.total_blocks - 8 * grouped_slots;
+    a.group = (int32_t)group;
+    a.grouped_slots = (int32_t)grouped_slots;
+    a.rest_per_xcd = (int32_t)((rest + 7) / 8);
+    plan->grid = (unsigned)((grouped_slots + a.rest_per_xcd) * 8);
+  }
   plan->lds_bytes = (size_t)br * a.pitch_bytes;
   return plan->lds_bytes <= 49152;
 }
