@@ -89,12 +89,14 @@ def test_tile_counts_around_the_number_of_compute_units(gpu_lib, oracle_lib, N, 
 # The resident-lhs kernel (one workgroup per compute unit, the lhs operands of each wavefront's K share copied to
 # LDS once, rhs dealt out in half tiles): at least one rhs tile per compute unit, more than 4 lhs rows, K of
 # 64 or 128 steps of 64 bytes. Tile counts that give the units whole tiles, half tiles at either end of their
-# ranges, and ranges of unequal length; lhs rows from one, two and four lhs tiles, fewer than 16 rows; a gap
+# ranges, ranges of unequal length, and equally many whole tiles per unit (dealt out in rounds instead of ranges); lhs rows from one, two and four lhs tiles, fewer than 16 rows; a gap
 # between rhs panels, strided lhs and out rows; with guard words around the output. int8 bit for bit.
 RESIDENT = [
     # flags, M, M0, N, K, K0
     (abi.MMT4D_TYPE_S8S8S32, 1, 16, 896, 64, 64),     # 64 steps; 3.5 tiles per unit
     (abi.MMT4D_TYPE_S8S8S32, 1, 16, 256, 128, 64),    # 128 steps; exactly one tile per unit
+    (abi.MMT4D_TYPE_S8S8S32, 1, 16, 768, 64, 64),     # three whole tiles per unit: one of every round of 256 tiles
+    (abi.MMT4D_TYPE_BF16BF16F32, 1, 16, 512, 512, 8),   # two whole tiles per unit, 128 steps
     (abi.MMT4D_TYPE_S8S8S32, 2, 8, 257, 256, 16),     # 64 steps; two lhs tiles of 8 rows
     (abi.MMT4D_TYPE_S8S8S32, 4, 4, 1000, 128, 32),    # 64 steps; four lhs tiles of 4 rows
     (abi.MMT4D_TYPE_S8S8S32, 3, 4, 511, 512, 16),     # 128 steps; 12 lhs rows
