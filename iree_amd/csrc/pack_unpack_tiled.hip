@@ -169,7 +169,7 @@ constexpr int kBlockBytes = 16384;  // bytes of the 2-D matrix per workgroup
 // rows). PL_BYTES: bytes of one contiguous LDS piece on the tiled side (16 when
 // 16 output bytes come from one LDS row, down to E for column access).
 //
-// LINE_ALIGNED (unpack of 4-byte elements into rows that do not start on
+// LINE_ALIGNED (unpack of 4-byte, and where rows are whole dwords apart 2-byte, elements into rows that do not start on
 // 128-byte lines, blocks one tile row tall): each row's piece of a block is
 // moved right to the next line boundary of THAT row, so a wavefront's 1 KiB
 // store is eight whole lines and no line is written in two parts by two
@@ -364,7 +364,7 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
     // few microseconds, and what it computes first is time with nothing in
     // flight. The columns around a block's edge are read by two blocks: those
     // loads leave their lines in the cache for the other one, the rest stream.
-    // A thread's vectors are 1024 elements apart, a whole number of tiles (the
+    // A thread's vectors are 256 vectors apart, a whole number of tiles (the
     // host sees to that): all of them are the same pieces of their tiles.
     typedef int v4 __attribute__((ext_vector_type(4)));
     const int32_t e0 = tid * VE, w0 = e0 & ((1 << log2_tile) - 1);
@@ -400,7 +400,7 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
     __syncthreads();
     // Whole lines: vector cv of row r starts s(r) + cv * EPV columns into the block.
     {
-      struct __attribute__((packed, aligned(E))) ShiftedVec {
+      struct __attribute__((packed, aligned(4))) ShiftedVec {  // (the host sees to it that shifts are whole dwords)
         uint32_t x, y, z, w;
       };
       FlatVec out[FLAT_PER_THREAD];
@@ -829,7 +829,9 @@ bool make_plan(const uint8_t* flat, const uint8_t* tiled, int64_t flat_stride0, 
   // Unpack of 4-byte elements into rows that are not whole 128-byte lines apart
   // (or do not start on one): every row's windows are moved to its own line
   // boundaries (tiled_kernel, LINE_ALIGNED).
-  plan->line_aligned = for_unpack && E == 4 && !tr_outer && flat_stride1 == 1 && size1 > bc && T0 * T1 <= 1024 &&
+  // (2-byte elements where the shifts are whole dwords; tiles that divide a thread's stride through the block.)
+  const bool dword_shifts = E == 4 || (E == 2 && (uintptr_t)flat % 4 == 0 && (size0 == 1 || (flat_stride0 * E) % 4 == 0));
+  plan->line_aligned = for_unpack && dword_shifts && !tr_outer && flat_stride1 == 1 && size1 > bc && T0 * T1 * E <= 4096 &&
                        ((uintptr_t)flat % 128 != 0 || (size0 > 1 && (flat_stride0 * E) % 128 != 0));
   a.ext_cols = 0;
   if (plan->line_aligned) a.ext_cols = (int32_t)(T1 > 128 / E ? T1 : 128 / E);
@@ -1157,13 +1159,16 @@ hipError_t launch_unpack(const UnpackArgs& original, hipStream_t stream, const c
   *name = "unpack_tiled";
   if (plan.line_aligned) {
     const dim3 grid(plan.grid), block(256);
-    if (plan.piece_bytes == 16) {
-      hipLaunchKernelGGL((tiled_kernel<4, 16, 16, true, true>), grid, block, plan.lds_bytes, stream, plan.args);
-    } else if (plan.piece_bytes == 8) {
-      hipLaunchKernelGGL((tiled_kernel<4, 16, 8, true, true>), grid, block, plan.lds_bytes, stream, plan.args);
+    void (*kernel)(const TiledArgs) = nullptr;
+    if (plan.elem_bytes == 4) {
+      kernel = plan.piece_bytes == 16 ? tiled_kernel<4, 16, 16, true, true>
+               : plan.piece_bytes == 8 ? tiled_kernel<4, 16, 8, true, true> : tiled_kernel<4, 16, 4, true, true>;
     } else {
-      hipLaunchKernelGGL((tiled_kernel<4, 16, 4, true, true>), grid, block, plan.lds_bytes, stream, plan.args);
+      kernel = plan.piece_bytes == 16 ? tiled_kernel<2, 16, 16, true, true>
+               : plan.piece_bytes == 8 ? tiled_kernel<2, 16, 8, true, true>
+               : plan.piece_bytes == 4 ? tiled_kernel<2, 16, 4, true, true> : tiled_kernel<2, 16, 2, true, true>;
     }
+    hipLaunchKernelGGL(kernel, grid, block, plan.lds_bytes, stream, plan.args);
     return hipGetLastError();
   }
   return launch_plan<true>(plan, stream);

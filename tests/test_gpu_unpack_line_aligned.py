@@ -1,4 +1,4 @@
-"""GPU parity for unpack of 4-byte elements into rows that do not start on
+"""GPU parity for unpack of 4-byte (and 2-byte) elements into rows that do not start on
 128-byte lines (unpack.c:190-247 is the semantics; tools/unpack_test.c draws
 such shapes all the time: any odd row length). The LDS-staged kernel then moves
 every row's windows to that row's own line boundaries, so a block stores
@@ -42,6 +42,15 @@ CASES = [
     (abi.UNPACK_TYPE_I32I32, 200, 70, 64, 1, 0, 0, 0),            # two blocks per row, the second 6 columns
     (abi.UNPACK_TYPE_F32F32, 19, 513, 2, 2, 0, 0, 0),             # small tiles, blocks of 2048 columns: one block per row
     (abi.UNPACK_TYPE_F32F32, 19, 4099, 2, 2, TI, 0, 0),
+    # 2-byte elements: rows a whole number of dwords apart take the same path, others the plain one.
+    (abi.UNPACK_TYPE_F16F16, 200, 8190, 16, 1, 0, 0, 0),
+    (abi.UNPACK_TYPE_BF16BF16, 77, 2 * 512 + 66, 16, 1, 0, 2, 6),
+    (abi.UNPACK_TYPE_F16F16, 77, 1100, 8, 8, 0, 0, 2),
+    (abi.UNPACK_TYPE_BF16BF16, 50, 3000, 16, 16, TI, 4, 0),
+    (abi.UNPACK_TYPE_F16F16, 40, 5000, 1, 16, 0, 0, 0),
+    (abi.UNPACK_TYPE_F16F16, 33, 700, 32, 8, TI, 0, 4),
+    (abi.UNPACK_TYPE_F16F16, 60, 2049, 16, 1, 0, 0, 0),          # odd row length: shifts of odd halfwords, plain path
+    (abi.UNPACK_TYPE_BF16BF16, 60, 2048, 16, 1, 0, 0, 3),        # odd offset
 ]
 
 
@@ -50,12 +59,11 @@ CASES = [
 def test_unpack_into_rows_off_the_cache_lines(gpu_lib, oracle_lib, case):
     typ, rows, cols, t0, t1, flags, row_gap, out_off = case
     e = abi.UNPACK_ELEM_BYTES[typ]
-    assert e == 4
     o0, o1 = -(-rows // t0), -(-cols // t1)
     s2, s3 = (t1, t0) if flags & TI else (t0, t1)
     in_stride0 = o1 * s2 * s3
     out_stride0 = cols + row_gap
-    in_off = 4
+    in_off = 16 // e
     src = synth.uniform_int8(61, 0, (in_off + o0 * in_stride0) * e)
     n_out = out_off + rows * out_stride0 + 64
 
