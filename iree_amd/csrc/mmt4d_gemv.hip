@@ -164,7 +164,10 @@ __global__ __launch_bounds__(64 * kWaves) void mmt4d_gemv_kernel(const GemvArgs 
 // LDS in wavefront order: results do not depend on scheduling.
 // Needs steps == kWaves * UNROLL (one batch of loads per wavefront and tile).
 template <int KIND, int kWaves, int UNROLL, int MAX_TILES>
-__global__ __launch_bounds__(64 * kWaves) void mmt4d_gemv_resident_lhs_kernel(const GemvArgs a) {
+// (The register budget is said explicitly: two buffers of UNROLL loads and MAX_TILES accumulators; left to its
+// own devices with 8 wavefronts the compiler takes all 256 registers for the shorter instantiation and still spills.)
+__global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(UNROLL >= 16 ? 2 : 3, UNROLL >= 16 ? 2 : 3)))
+void mmt4d_gemv_resident_lhs_kernel(const GemvArgs a) {
   typedef typename Acc<KIND>::type acc_t;
   extern __shared__ uint4 gemv_lds[];  // [kWaves][UNROLL][64] lhs operands; then [MAX_TILES][kWaves][64] partial sums
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -203,15 +206,17 @@ __global__ __launch_bounds__(64 * kWaves) void mmt4d_gemv_resident_lhs_kernel(co
     if (u == tiles - 1 && skip_high_half_of_last && row >= 8) return false;
     return true;
   };
+  // (Lanes whose rows of a half tile belong to another unit load nothing and keep what they held: rhs row n only
+  // ever reaches column n of the result, and those columns are not stored.)
   uint4 r[2][UNROLL];
+#pragma unroll
+  for (int s = 0; s < UNROLL; ++s) r[0][s] = r[1][s] = make_uint4(0, 0, 0, 0);
   auto fetch = [&](int u, uint4* dst) {
     const uint8_t* p = rhs_lane + tile_of(u) * a.rhs_stride_bytes;
     const bool loaded = tile_rows_loaded(u);
 #pragma unroll
-    for (int s = 0; s < UNROLL; ++s) {
-      dst[s] = make_uint4(0, 0, 0, 0);
+    for (int s = 0; s < UNROLL; ++s)
       if (loaded) dst[s] = __builtin_bit_cast(uint4, __builtin_nontemporal_load((const v4i32*)(p + s * rhs_step_bytes)));
-    }
   };
   fetch(0, r[0]);
   uint4* own_lhs = gemv_lds + (wave * UNROLL) * 64 + lane;
@@ -274,6 +279,17 @@ __device__ __forceinline__ uint4 widen_i4_times16(uint32_t lo, uint32_t hi) {
   return r;
 }
 
+// The same without the interleaving: the even elements of each dword, then the
+// odd ones (6 instructions instead of 10). For products with an lhs operand whose
+// bytes are in the same order (lhs_bytes_even_then_odd).
+__device__ __forceinline__ uint4 widen_i4_times16_even_then_odd(uint32_t lo, uint32_t hi) {
+  return make_uint4((lo << 4) & 0xF0F0F0F0u, lo & 0xF0F0F0F0u, (hi << 4) & 0xF0F0F0F0u, hi & 0xF0F0F0F0u);
+}
+__device__ __forceinline__ uint4 lhs_bytes_even_then_odd(uint4 v) {
+  return make_uint4(__builtin_amdgcn_perm(v.y, v.x, 0x06040200u), __builtin_amdgcn_perm(v.y, v.x, 0x07050301u),
+                    __builtin_amdgcn_perm(v.w, v.z, 0x06040200u), __builtin_amdgcn_perm(v.w, v.z, 0x07050301u));
+}
+
 // s8s4s32 for a skinny lhs: the int4 rhs streams at half a byte per weight.
 // One step covers 128 values of K. Lane l (row l & 15, g = l >> 4) loads the 16
 // bytes = 32 nibbles of its rhs row at K values 32*g .. 32*g + 31 of the step
@@ -323,14 +339,17 @@ __global__ __launch_bounds__(64 * kWaves) void mmt4d_gemv_i4_kernel(const GemvAr
                                                    __builtin_bit_cast(v4i32, l1), acc[t], 0, 0, 0);
   };
   int32_t s = s_begin;
+  // (Lanes of lhs rows that do not exist never load: their operands stay zero, set once.)
+  uint4 l0[UNROLL], l1[UNROLL];
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) l0[u] = l1[u] = make_uint4(0, 0, 0, 0);
   for (; s + UNROLL <= s_end; s += UNROLL) {
-    uint4 r[UNROLL][TN], l0[UNROLL], l1[UNROLL];
+    uint4 r[UNROLL][TN];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
 #pragma unroll
       for (int t = 0; t < TN; ++t)
         r[u][t] = __builtin_bit_cast(uint4, __builtin_nontemporal_load((const v4i32*)(rhs_lane[t] + (int64_t)(s + u) * 1024)));
-      l0[u] = l1[u] = make_uint4(0, 0, 0, 0);
       if (lhs_valid) {
         l0[u] = *(const uint4*)(lhs_lane + (s + u) * lhs_step_bytes);
         l1[u] = *(const uint4*)(lhs_lane + (s + u) * lhs_step_bytes + 16);
@@ -374,7 +393,8 @@ __global__ __launch_bounds__(64 * kWaves) void mmt4d_gemv_i4_kernel(const GemvAr
 // workgroup per compute unit, wavefront w keeps the lhs operands of its K share (two 16-byte pieces per lane
 // and step) in LDS and streams the unit's half tiles past them. Needs steps == kWaves * UNROLL.
 template <int kWaves, int UNROLL, int MAX_TILES>
-__global__ __launch_bounds__(64 * kWaves) void mmt4d_gemv_i4_resident_lhs_kernel(const GemvArgs a) {
+__global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(4, 4)))  // (128 registers, as with 16 wavefronts)
+void mmt4d_gemv_i4_resident_lhs_kernel(const GemvArgs a) {
   extern __shared__ uint4 gemv_lds[];  // [kWaves][UNROLL][2][64] lhs operands; then [MAX_TILES][kWaves][64] partial sums
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int row = lane & 15, g = lane >> 4;
@@ -407,15 +427,18 @@ __global__ __launch_bounds__(64 * kWaves) void mmt4d_gemv_i4_resident_lhs_kernel
   };
   // Loads of up to DEPTH - 1 tiles in flight ahead of the one being multiplied (8 KiB per wavefront and tile).
   constexpr int DEPTH = 4;
+  // (Lanes whose rows of a half tile belong to another unit load nothing and keep what they held, see above.)
   uint4 r[DEPTH][UNROLL];
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d)
+#pragma unroll
+    for (int s = 0; s < UNROLL; ++s) r[d][s] = make_uint4(0, 0, 0, 0);
   auto fetch = [&](int u, uint4* dst) {
     const uint8_t* p = rhs_lane + (int64_t)u * a.rhs_stride_bytes;
     const bool loaded = tile_rows_loaded(u);
 #pragma unroll
-    for (int s = 0; s < UNROLL; ++s) {
-      dst[s] = make_uint4(0, 0, 0, 0);
+    for (int s = 0; s < UNROLL; ++s)
       if (loaded) dst[s] = __builtin_bit_cast(uint4, __builtin_nontemporal_load((const v4i32*)(p + (int64_t)s * 1024)));
-    }
   };
 #pragma unroll
   for (int u = 0; u < DEPTH - 1; ++u)
@@ -433,8 +456,9 @@ __global__ __launch_bounds__(64 * kWaves) void mmt4d_gemv_i4_resident_lhs_kernel
     }
 #pragma unroll
     for (int s = 0; s < UNROLL; ++s) {
-      own_lhs[s * 128] = l0[s];
-      own_lhs[s * 128 + 64] = l1[s];
+      // (bytes reordered once, here, so that the nibbles need no interleaving in the loop)
+      own_lhs[s * 128] = lhs_bytes_even_then_odd(l0[s]);
+      own_lhs[s * 128 + 64] = lhs_bytes_even_then_odd(l1[s]);
     }
   }
 
@@ -448,9 +472,9 @@ __global__ __launch_bounds__(64 * kWaves) void mmt4d_gemv_i4_resident_lhs_kernel
 #pragma unroll
       for (int s = 0; s < UNROLL; ++s) {
         const uint4 w = r[u % DEPTH][s];
-        acc[u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i32, widen_i4_times16(w.x, w.y)),
+        acc[u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i32, widen_i4_times16_even_then_odd(w.x, w.y)),
                                                        __builtin_bit_cast(v4i32, own_lhs[s * 128]), acc[u], 0, 0, 0);
-        acc[u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i32, widen_i4_times16(w.z, w.w)),
+        acc[u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i32, widen_i4_times16_even_then_odd(w.z, w.w)),
                                                        __builtin_bit_cast(v4i32, own_lhs[s * 128 + 64]), acc[u], 0, 0, 0);
       }
     }
@@ -585,11 +609,13 @@ hipError_t launch_gemv(const Mmt4dArgs& a, hipStream_t stream, const char** name
   if (!make_args(a, false, &kind, &g)) return hipErrorInvalidValue;
   *name = "mmt4d_gemv";
   if (kind == kI8I4) {
-    // More than 4 lhs rows and a tile or more per compute unit: the resident-lhs kernel, where its instantiations
-    // fit the number of steps (each of 128 values of K; the lhs of 64 steps fills 128 KiB of LDS).
+    // More than 4 lhs rows and a tile or more per compute unit, or six tiles or more per unit with any number of
+    // rows (28672 x 8192, one row: 0.69 -> 0.71 of the HBM peak; at 3.5 tiles per unit the kernel below is ahead,
+    // 0.51 against 0.48): the resident-lhs kernel, where its instantiations fit the number of steps (each of 128
+    // values of K; the lhs of 64 steps fills 128 KiB of LDS).
     const int units = compute_units();
     constexpr int MAX_TILES = 8;
-    if ((g.M << g.log2_M0) > 4 && units > 0 && g.N >= units && (2 * (int64_t)g.N + units - 1) / units / 2 + 1 <= MAX_TILES &&
+    if (((g.M << g.log2_M0) > 4 || g.N >= 6 * (int64_t)units) && units > 0 && g.N >= units && (2 * (int64_t)g.N + units - 1) / units / 2 + 1 <= MAX_TILES &&
         (g.steps == 64 || g.steps == 32)) {
       const int lds_bytes = 128 * 1024;  // the lhs operands of 64 steps; the partial sums need less
       // (16 wavefronts x 4 steps with three tiles' loads in flight: 0.65 of the HBM peak at 16 x 28672 x 8192 against

@@ -30,11 +30,17 @@ CASES = [
     (1, 16, 18, 8, 16, None),                 # 8-byte rhs row pieces
     (1, 2, 18, 2048, 64, b"mmt4d_gemv"),      # K * K0 = 131072: 16x-scaled sums could overflow; chained over two slices of K
     # The resident-lhs kernel: more than 4 lhs rows, a tile or more per compute unit, 64 or 32 steps of 128 values.
+    # (Its lhs operands sit in LDS with the bytes of every dword pair reordered to match nibbles that are widened
+    # without interleaving: any lhs value pattern must still come out bit for bit.)
     (1, 16, 897, 256, 32, b"mmt4d_gemv_resident_lhs"),    # K = 8192: half tiles at both ends of the units' ranges
     (1, 16, 256, 128, 64, b"mmt4d_gemv_resident_lhs"),    # one tile per unit, K0 = 64
     (2, 8, 1791, 128, 32, b"mmt4d_gemv_resident_lhs"),    # K = 4096 (32 steps), two lhs tiles, up to 7 tiles per unit
     (3, 4, 300, 256, 32, b"mmt4d_gemv_resident_lhs"),     # 12 lhs rows
     (1, 16, 2000, 256, 32, b"mmt4d_gemv"),                # more tiles per unit than it keeps accumulators for
+    # Six tiles or more per compute unit: the resident-lhs kernel with any number of lhs rows.
+    (1, 1, 1600, 128, 32, b"mmt4d_gemv_resident_lhs"),    # one lhs row, 32 steps
+    (1, 4, 1537, 128, 64, b"mmt4d_gemv_resident_lhs"),    # four lhs rows, 64 steps, half tiles in play
+    (1, 2, 1535, 128, 32, b"mmt4d_gemv"),                 # just under six tiles per unit
 ]
 
 
