@@ -620,7 +620,8 @@ __device__ __forceinline__ void wait_loads_but() {
 // explicitly, because left to its occupancy heuristics the compiler may keep
 // the accumulators in scratch memory instead.)
 // STAGGER: 0 = every accumulator stored after the last MFMA; 1 = staggered tail (see below); 2 = the same for
-// an accumulating call.
+// an accumulating call, the destination read in the tail; 3 = accumulating call with the destination read and
+// added during the main loop (needs enough steps), tail as in 1.
 template <int KIND, bool RHS_I4, bool NARROW, int G, int AM, int BN, int STAGES, int STAGGER = 0>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, AM * BN >= 16 ? 1 : (AM * BN >= 4 ? 2 : 4))))
 void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
@@ -957,7 +958,11 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
   // load per MFMA. The reads end a quarter of the step before its end, so that
   // the last of them has returned when the next step starts; fragments are
   // read in the order the next step consumes them.
-  auto step = [&](const uint4 (*cur_a)[2], const uint4 (*cur_b)[2], uint4 (*nxt_a)[2], uint4 (*nxt_b)[2]) {
+  // (`held_loads_behind`: the eight loads of destination values that variant 3 issues at the start of a phase
+  // are younger than the chunk this step waits for, and may stay in flight with it.)
+  // `between_mfmas(m)`: extra work placed behind MFMA m of the step (variant 3 adds destination values there).
+  auto step_with = [&](const uint4 (*cur_a)[2], const uint4 (*cur_b)[2], uint4 (*nxt_a)[2], uint4 (*nxt_b)[2],
+                       bool held_loads_behind, auto between_mfmas) {
     constexpr int SUB = SubSteps<KIND>::value;
     constexpr int MFMAS = 2 * AM * BN * SUB;
     // Units a fragment's LDS reads are dealt out in: a 128-bit read; two pairs of
@@ -1013,9 +1018,16 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
       acc[i][j] = mfma<KIND>(cur_b[j][kk], cur_a[i][kk], acc[i][j], sub);
     };
 #pragma unroll
-    for (int m = 0; m < LEAD; ++m) multiply(m);
+    for (int m = 0; m < LEAD; ++m) {
+      multiply(m);
+      between_mfmas(m);
+    }
     __builtin_amdgcn_sched_barrier(0);
-    wait_loads_but<LOADS*(AHEAD - 2)>();
+    if constexpr (STAGGER == 3) {
+      if (held_loads_behind) wait_loads_but<LOADS*(AHEAD - 2) + 8>(); else wait_loads_but<LOADS*(AHEAD - 2)>();
+    } else {
+      wait_loads_but<LOADS*(AHEAD - 2)>();
+    }
     __builtin_amdgcn_s_barrier();
     // The fragments read during this step are those of chunk load_chunk - AHEAD + 1.
     const bool cut_next = cut_bytes != 0 && load_chunk - AHEAD + 1 == last_chunk;
@@ -1089,6 +1101,7 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
       }
       split_units_of(slot - SPLIT_DELAY);
       multiply(m);
+      between_mfmas(m);
       if (m == MFMAS - 1) {
         // Advance the running state (clamped at the last chunk: the loads
         // issued beyond it are redundant, their stages are never read).
@@ -1123,6 +1136,10 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
         }
       }
     }
+  };
+  auto step = [&](const uint4 (*cur_a)[2], const uint4 (*cur_b)[2], uint4 (*nxt_a)[2], uint4 (*nxt_b)[2],
+                  bool held_loads_behind = false) {
+    step_with(cur_a, cur_b, nxt_a, nxt_b, held_loads_behind, [](int) {});
   };
 
   // The last AHEAD chunks, for the 256x256 tile. At the end of the loop above
@@ -1390,6 +1407,66 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
         for (int j = 0; j < BN; ++j) pb[j][kk] = qb[j][kk];
       }
       kc = 1;
+    }
+    if constexpr (STAGGER == 3) {
+      // An accumulating call: what the destination held is added to the accumulators on the way, so that the
+      // tail only stores (read in the tail, the 256 KiB per workgroup come from HBM on top of the stores, with
+      // three chunks of MFMAs to hide under). One phase per pair of fragments: its eight quads are loaded, an even
+      // number of steps runs, and in the last of them the values are added, each fragment's behind its first
+      // MFMA of that step, two registers per MFMA, done before its second. The loads are issued from assembly,
+      // like those of the ring, so that the compiler does not wait for them (its waits would be for every load
+      // in flight, the ring's youngest included): after three steps they have landed, because loads return in
+      // order and the third step waits for a chunk that was requested after them. A lane outside the matrix loads
+      // from the start of the destination; what it adds is never stored.
+      static_assert(SubSteps<KIND>::value == 1, "one MFMA per fragment and K-step");
+      const OutAddressing o = out_addressing();
+      constexpr int PAIRS = AM * (BN / 2);
+      // The workgroups of a launch run in step; were all of them to load a pair at the same moment, the 16 MiB
+      // would take longer to arrive than the two steps the ring can wait. Each therefore starts its phases a
+      // different number of steps into the loop (one phase's worth of steps is set aside for that).
+      const int per_phase = ((main_steps - kc) / (PAIRS + 1)) & ~1;  // (the host sees to it that this is at least 4)
+      for (int lead = 2 * ((int)((blockIdx.x >> 3) & 7) * (per_phase / 2) >> 3); lead > 0; lead -= 2, kc += 2) {
+        step(pa, pb, qa, qb);
+        step(qa, qb, pa, pb);
+      }
+#pragma unroll
+      for (int pair = 0; pair < PAIRS; ++pair) {
+        const int i = pair / (BN / 2), jp = pair % (BN / 2);
+        bool row_inside;
+        const uint8_t* row_out = out_row_pointer(o, i, &row_inside);
+        out_stored_t held[8];
+#pragma unroll
+        for (int n = 0; n < 8; ++n) {
+          const int j = 2 * jp + n / 4, q = n % 4;
+          const uint8_t* from = row_inside && (o.col_inside >> (4 * j + q) & 1) ? row_out + o.col_off[j][q] : a.out;
+          if constexpr (NARROW) asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(held[n]) : "v"(from) : "memory");
+          else asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(held[n]) : "v"(from) : "memory");
+        }
+        int held_loads_behind = 1;
+        for (int s = 0; s + 2 < per_phase; s += 2, kc += 2) {
+          asm volatile("" : "+s"(held_loads_behind));  // (one copy of the loop body, not a peeled first pass)
+          step(pa, pb, qa, qb, held_loads_behind != 0);
+          step(qa, qb, pa, pb, held_loads_behind != 0);
+          held_loads_behind = 0;
+        }
+        step(pa, pb, qa, qb);
+        out_quad_t was[8];
+#pragma unroll
+        for (int n = 0; n < 8; ++n) {
+          asm volatile("" : "+v"(held[n]));
+          was[n] = out_to_float(held[n]);
+        }
+        step_with(qa, qb, pa, pb, false, [&](int m) {
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            const int j = 2 * jp + t, slot = m - (i * BN + j + 2);
+            if (slot < 0 || slot >= 8) continue;
+#pragma unroll
+            for (int r = 2 * slot; r < 2 * slot + 2; ++r) acc[i][j][r] += was[4 * t + r / 4][r % 4];
+          }
+        });
+        kc += 2;
+      }
     }
     for (; kc + 1 < main_steps; kc += 2) {
       step(pa, pb, qa, qb);
@@ -1690,7 +1767,9 @@ hipError_t launch_direct(MfmaArgs m, hipStream_t stream, bool staggered_tail = t
   // The 256x256 tile with the staggered tail: K in whole chunks, enough of them.
   if constexpr (AM == 4 && BN == 4 && !RHS_I4 && G != 2 && KIND != kF32) {
     if (staggered_tail && ((int64_t)m.K * m.lhs_rb) % 64 == 0 && m.chunks >= 2 * STAGES) {
-      if (m.accumulate) kernel = mmt4d_mfma_direct_kernel<KIND, RHS_I4, NARROW, G, AM, BN, STAGES, 2>;
+      // (Accumulating: read the destination during the loop where every one of the eight phases gets four steps.)
+      if (m.accumulate && m.chunks >= STAGES + 9 * 4) kernel = mmt4d_mfma_direct_kernel<KIND, RHS_I4, NARROW, G, AM, BN, STAGES, 3>;
+      else if (m.accumulate) kernel = mmt4d_mfma_direct_kernel<KIND, RHS_I4, NARROW, G, AM, BN, STAGES, 2>;
       else kernel = mmt4d_mfma_direct_kernel<KIND, RHS_I4, NARROW, G, AM, BN, STAGES, 1>;
     }
   }

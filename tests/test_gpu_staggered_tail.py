@@ -36,6 +36,16 @@ CASES = [
     (F16, 3584, 3584, 16, 16, 16, 18),    # 9 chunks of 32 halves
     (BF16, 3520, 3616, 16, 16, 8, 40),    # 10 chunks
     (F16F16 | SKIP, 3584, 3584, 16, 16, 16, 16),   # 16-bit output, one rounding at the end
+    # 36 chunks and more: an accumulating call reads the destination during the main loop, a pair of fragments per
+    # phase, instead of in the tail.
+    (S8, 3584, 3584, 8, 8, 4, 576),       # 36 chunks: the fewest (an odd number of main steps, four per phase)
+    (S8, 3500, 3600, 8, 8, 4, 592),       # 37 chunks, rows and columns end inside a block tile
+    (S8, 3584, 3584, 16, 16, 64, 45),     # 45 chunks: steps left over after the eight phases
+    (S8, 3501, 3584, 1, 16, 64, 40),      # row-major lhs and result
+    (S8, 3584, 3584, 8, 8, 1, 2432),      # 1-byte row pieces, 38 chunks
+    (F16, 3584, 3584, 16, 16, 16, 80),    # 40 chunks
+    (BF16, 3520, 3616, 16, 16, 8, 200),   # 50 chunks, ragged
+    (F16F16 | SKIP, 3584, 3584, 16, 16, 16, 76),   # 16-bit output: 8-byte quads
 ]
 
 
