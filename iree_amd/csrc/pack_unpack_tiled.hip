@@ -185,7 +185,7 @@ constexpr int kBlockBytes = 16384;  // bytes of the 2-D matrix per workgroup
 // requested on the tiled side cost what is left, whether or not the loads are
 // masked down to the rows that are used, and although the lines shared by two
 // blocks come from HBM only once.
-template <int E, int W, int PL_BYTES, bool UNPACK, bool LINE_ALIGNED = false>
+template <int E, int W, int PL_BYTES, bool UNPACK, int LINE_ALIGNED = 0>  // (1: line-aligned unpack, 2: the same with an outer transpose)
 __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
   static_assert(!LINE_ALIGNED || (UNPACK && W == 16), "line-aligned windows are for unpack");
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -348,7 +348,7 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
   };
 
   if constexpr (LINE_ALIGNED) {
-    constexpr int MAX_TILED = TILED_PER_THREAD + 4;
+    constexpr int MAX_TILED = TILED_PER_THREAD + (LINE_ALIGNED == 2 ? 2 : 4);  // (the host keeps to these)
     const int32_t bc = 1 << a.log2_bc;
     const int32_t log2_tile = a.log2_t0 + a.log2_t1;
     const bool first_block = block1 == 0;
@@ -372,6 +372,38 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
     const int32_t total_vecs = ((bc + a.ext_cols) << a.log2_br) / VE;
     TiledVec regs[MAX_TILED];
     bool wanted[MAX_TILED];
+    if constexpr (LINE_ALIGNED == 2) {
+      // Outer transpose: the tiled side is one run per tile column, and the columns after the block's own
+      // are further runs; the block's enumeration simply goes on (tiled_coord).
+      TiledCoord first[MAX_TILED];
+#pragma unroll
+      for (int u = 0; u < MAX_TILED; ++u) {
+        const int32_t vec = tid + 256 * u;
+        first[u] = tiled_coord(a, vec * VE, tile0_base, tile1_base);
+        wanted[u] = vec < total_vecs && first[u].in_range;
+        if (wanted[u]) {
+          const uint8_t* g = a.src + first[u].global_elem * E;
+          if (first[u].col < 128 / E || first[u].col >= bc)
+            regs[u].vec = *(const uint4*)g;
+          else
+            regs[u].vec = __builtin_bit_cast(uint4, __builtin_nontemporal_load((const v4*)g));
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < MAX_TILED; ++u) {
+        if (!wanted[u]) continue;
+#pragma unroll
+        for (int q = 0; q < PIECES; ++q) {
+          int32_t row = first[u].row, col = first[u].col;
+          if (q > 0) {
+            const TiledCoord c = tiled_coord(a, (tid + 256 * u) * VE + q * PL, tile0_base, tile1_base);
+            row = c.row;
+            col = c.col;
+          }
+          *(piece_t*)(lds + row * a.pitch_bytes + col * E) = regs[u].piece[q];
+        }
+      }
+    } else {
 #pragma unroll
     for (int u = 0; u < MAX_TILED; ++u) {
       const int32_t vec = tid + 256 * u, o1l = (vec * VE) >> log2_tile, col0 = o1l << a.log2_t1;
@@ -396,6 +428,7 @@ __global__ __launch_bounds__(256) void tiled_kernel(const TiledArgs a) {
       const int32_t o1l = ((tid + 256 * u) * VE) >> log2_tile;
 #pragma unroll
       for (int q = 0; q < PIECES; ++q) *(piece_t*)(lds + lds_base[q] + ((o1l << a.log2_t1) * E)) = regs[u].piece[q];
+    }
     }
     __syncthreads();
     // Whole lines: vector cv of row r starts s(r) + cv * EPV columns into the block.
@@ -831,10 +864,11 @@ bool make_plan(const uint8_t* flat, const uint8_t* tiled, int64_t flat_stride0, 
   // boundaries (tiled_kernel, LINE_ALIGNED).
   // (2-byte elements where the shifts are whole dwords; tiles that divide a thread's stride through the block.)
   const bool dword_shifts = E == 4 || (E == 2 && (uintptr_t)flat % 4 == 0 && (size0 == 1 || (flat_stride0 * E) % 4 == 0));
-  plan->line_aligned = for_unpack && dword_shifts && !tr_outer && flat_stride1 == 1 && size1 > bc && T0 * T1 * E <= 4096 &&
+  plan->line_aligned = for_unpack && dword_shifts && flat_stride1 == 1 && size1 > bc && T0 * T1 * E <= 4096 &&
                        ((uintptr_t)flat % 128 != 0 || (size0 > 1 && (flat_stride0 * E) % 128 != 0));
   a.ext_cols = 0;
   if (plan->line_aligned) a.ext_cols = (int32_t)(T1 > 128 / E ? T1 : 128 / E);
+  if (plan->line_aligned && tr_outer && a.ext_cols * br * E / 16 > 512) plan->line_aligned = false, a.ext_cols = 0;
   a.pitch_bytes = choose_pitch(a, E, piece, a.ext_cols);
   a.blocks1 = (int32_t)((size1 + bc - 1) / bc);
   // Blocks must cover every tile of the tiled side, not only the 2-D extent
@@ -1160,14 +1194,13 @@ hipError_t launch_unpack(const UnpackArgs& original, hipStream_t stream, const c
   if (plan.line_aligned) {
     const dim3 grid(plan.grid), block(256);
     void (*kernel)(const TiledArgs) = nullptr;
-    if (plan.elem_bytes == 4) {
-      kernel = plan.piece_bytes == 16 ? tiled_kernel<4, 16, 16, true, true>
-               : plan.piece_bytes == 8 ? tiled_kernel<4, 16, 8, true, true> : tiled_kernel<4, 16, 4, true, true>;
-    } else {
-      kernel = plan.piece_bytes == 16 ? tiled_kernel<2, 16, 16, true, true>
-               : plan.piece_bytes == 8 ? tiled_kernel<2, 16, 8, true, true>
-               : plan.piece_bytes == 4 ? tiled_kernel<2, 16, 4, true, true> : tiled_kernel<2, 16, 2, true, true>;
-    }
+#define UK_LINE_ALIGNED_KERNEL(E, MODE)                                                                        \
+  (plan.piece_bytes == 16 ? tiled_kernel<E, 16, 16, true, MODE>                                                 \
+   : plan.piece_bytes == 8 ? tiled_kernel<E, 16, 8, true, MODE>                                                 \
+   : (plan.piece_bytes == 4 || E == 4) ? tiled_kernel<E, 16, 4, true, MODE> : tiled_kernel<E, 16, E, true, MODE>)
+    if (plan.elem_bytes == 4) kernel = tr_outer ? UK_LINE_ALIGNED_KERNEL(4, 2) : UK_LINE_ALIGNED_KERNEL(4, 1);
+    else kernel = tr_outer ? UK_LINE_ALIGNED_KERNEL(2, 2) : UK_LINE_ALIGNED_KERNEL(2, 1);
+#undef UK_LINE_ALIGNED_KERNEL
     hipLaunchKernelGGL(kernel, grid, block, plan.lds_bytes, stream, plan.args);
     return hipGetLastError();
   }

@@ -22,7 +22,7 @@ from test_gpu_configs import gpu_lib  # noqa: F401
 
 pytestmark = pytest.mark.gpu
 
-TI = abi.UNPACK_TRANSPOSE_INNER
+TI, TO = abi.UNPACK_TRANSPOSE_INNER, abi.UNPACK_TRANSPOSE_OUTER
 
 CASES = [
     # type, rows, cols, tile rows, tile cols, flags, row gap (elements), out offset (elements)
@@ -51,6 +51,14 @@ CASES = [
     (abi.UNPACK_TYPE_F16F16, 33, 700, 32, 8, TI, 0, 4),
     (abi.UNPACK_TYPE_F16F16, 60, 2049, 16, 1, 0, 0, 0),          # odd row length: shifts of odd halfwords, plain path
     (abi.UNPACK_TYPE_BF16BF16, 60, 2048, 16, 1, 0, 0, 3),        # odd offset
+    # Outer transposes: the tiled side is one run per tile column, the columns after the block's own are further runs.
+    (abi.UNPACK_TYPE_F32F32, 300, 2 * 256 + 200, 16, 1, TO, 0, 0),
+    (abi.UNPACK_TYPE_F32F32, 300, 1025, 16, 16, TO, 1, 3),
+    (abi.UNPACK_TYPE_I32I32, 130, 1300, 8, 8, TO | TI, 0, 5),
+    (abi.UNPACK_TYPE_F32F32, 77, 3 * 256 + 31, 1, 16, TO, 2, 0),
+    (abi.UNPACK_TYPE_F32F32, 200, 600, 64, 4, TO | TI, 0, 0),
+    (abi.UNPACK_TYPE_F16F16, 300, 2 * 512 + 66, 16, 16, TO, 0, 2),
+    (abi.UNPACK_TYPE_BF16BF16, 140, 5000, 16, 1, TO | TI, 2, 0),
 ]
 
 
@@ -60,11 +68,12 @@ def test_unpack_into_rows_off_the_cache_lines(gpu_lib, oracle_lib, case):
     typ, rows, cols, t0, t1, flags, row_gap, out_off = case
     e = abi.UNPACK_ELEM_BYTES[typ]
     o0, o1 = -(-rows // t0), -(-cols // t1)
+    s0, s1 = (o1, o0) if flags & TO else (o0, o1)
     s2, s3 = (t1, t0) if flags & TI else (t0, t1)
-    in_stride0 = o1 * s2 * s3
+    in_stride0 = s1 * s2 * s3
     out_stride0 = cols + row_gap
     in_off = 16 // e
-    src = synth.uniform_int8(61, 0, (in_off + o0 * in_stride0) * e)
+    src = synth.uniform_int8(61, 0, (in_off + s0 * in_stride0) * e)
     n_out = out_off + rows * out_stride0 + 64
 
     def params(src_ptr, dst_ptr):
@@ -73,7 +82,7 @@ def test_unpack_into_rows_off_the_cache_lines(gpu_lib, oracle_lib, case):
         p.in_offset, p.out_offset = in_off, out_off
         p.in_stride0, p.in_stride1 = in_stride0, s2 * s3
         p.out_stride0, p.out_stride1 = out_stride0, 1
-        p.in_size0, p.in_size1, p.in_size2, p.in_size3 = o0, o1, s2, s3
+        p.in_size0, p.in_size1, p.in_size2, p.in_size3 = s0, s1, s2, s3
         p.out_size0, p.out_size1 = rows, cols
         p.flags = typ | flags
         return p
