@@ -1095,11 +1095,11 @@ hipError_t launch_pack(const PackArgs& original, hipStream_t stream, const char*
     a.out_size2 = 1;
     tr_inner = true;
   }
-  // The other way round for 4-byte elements: a tile one ROW tall stored
-  // inner-transposed ([T1][1]) is that row's T1 consecutive elements, i.e. the
-  // untransposed [1][T1]; as such its 16-byte vectors are whole pieces of a
-  // row in LDS instead of four separate elements.
-  if (tr_inner && a.out_size3 == 1 && a.elem_bytes == 4) {
+  // The other way round: a tile one ROW tall stored inner-transposed ([T1][1])
+  // is that row's T1 consecutive elements, i.e. the untransposed [1][T1]; as
+  // such its 16-byte vectors are whole pieces of a row in LDS instead of
+  // separate elements (int8 [16383, 16382] into 1x16 tiles: 3.6 -> 5.4 TB/s).
+  if (tr_inner && a.out_size3 == 1) {
     a.out_size3 = a.out_size2;
     a.out_size2 = 1;
     tr_inner = false;
