@@ -1030,7 +1030,9 @@ void mmt4d_mfma_direct_kernel(const MfmaArgs a) {
     }
     __builtin_amdgcn_s_barrier();
     // The fragments read during this step are those of chunk load_chunk - AHEAD + 1.
-    const bool cut_next = cut_bytes != 0 && load_chunk - AHEAD + 1 == last_chunk;
+    // (The variants with the staggered tail are launched for K in whole chunks only: nothing to cut there, and the
+    // masking, which the compiler makes unconditional, 64 instructions per step, is left out.)
+    const bool cut_next = STAGGER == 0 && cut_bytes != 0 && load_chunk - AHEAD + 1 == last_chunk;
     const uint8_t* read_a = ring_bytes + read_stage_off + frag_a_off + pair_a_lane;
     const uint8_t* read_a_kk1 = read_a + lhs_kk1_step;  // (used where the lhs has 16-byte pieces)
     const uint8_t* read_b = ring_bytes + read_stage_off + frag_b_off + pair_b_lane;
