@@ -970,7 +970,7 @@ def main():
 
     head = _headline(torch, lib, abi, synth, args.steps, args.warmup)
     sustained = _sustained_ceiling(torch, abi, synth)
-    also = None if args.no_also else _also(torch, lib, abi, synth, max(6, args.steps // 5), 2)
+    also = None if args.no_also else _also(torch, lib, abi, synth, max(6, args.steps // 5), 5)
     lib.iree_uk_mi355x_set_stream(None, 0)
     if also is not None:
         # The same call the way the reference's callers make it: host pointers,
