@@ -103,6 +103,15 @@ static inline void wait_for_all_loads_but(int n) {
 #undef WAIT_CASE
 }
 
+// The compiler keeps its own count of the loads it has issued and waits for
+// a loaded register at its first use. It does not see the loads issued by the
+// inline assembly above, and the counter completes in order: a first use of
+// the loaded accumulators inside the K loop becomes a wait in every trip, which
+// then also waits for the tile loads issued moments before and so undoes the
+// ring. An empty statement that uses the accumulators puts that wait in front
+// of the loop instead, once.
+static inline void accumulators_have_arrived(int32x4_t *c) { __asm__ volatile("" : "+a"(*c)); }
+
 // A pointer that is the same in every lane, said so to the compiler.
 static inline const int32x4_t *wavefront_uniform(const int32x4_t *p) {
   const uint64_t bits = (uint64_t)p;
@@ -214,6 +223,9 @@ static inline void issue_tile_loads(uint32_t lds_address, const int32x4_t *tile_
     }
     wait_for_all_loads_but((ahead - 1) * loads);
     workgroup_barrier();
+  }
+  for (int m = 0; m < intrinsics_m; ++m) {
+    for (int n = 0; n < intrinsics_n; ++n) accumulators_have_arrived(&c_regs[m][n]);
   }
 
   // The buffer being read and the buffer being filled.
