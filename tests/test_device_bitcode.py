@@ -78,3 +78,42 @@ int main(void) {
     # 128x128: 16 KiB per step, ring kept within 32 KiB: 2 buffers; only B staged (256 vectors = 4 KiB): 4 buffers;
     # only A staged (2*64 vectors = 2 KiB): 4 buffers; one subgroup: nothing; narrow A (64 vectors = 1 KiB): 4.
     assert got == [131072, 131072, 32768, 16384, 8192, 0, 4096]
+
+
+def test_k_loop_of_an_inlined_microkernel_waits_only_where_the_microkernel_says(tmp_path):
+    # The tile loads are inline assembly, which the compiler's own load counting does not see, and the load
+    # counter completes in order: a wait the compiler places inside the K loop (for the accumulators it loaded
+    # before the loop, at their first use) would in every trip also wait for the tile loads issued moments
+    # before, and the ring of buffers would never run ahead. Compile the wrapper the way the package does and
+    # look at the loop of the 256x256 instantiation: every wait on the load counter in it comes from the
+    # microkernel's assembly statements.
+    bc = str(tmp_path / (NAME + ".gfx950.bc"))
+    cmd = [hip_build.CLANG] + hip_build.BITCODE_FLAGS + [os.path.join(hip_build.DEVICE_DIR, NAME + ".c"), "-o", bc]
+    subprocess.run(cmd, check=True, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+    asm = str(tmp_path / "multi_mma.s")
+    cmd = [hip_build.HIPCC] + hip_build.COMMON_FLAGS + [
+        "-Xclang", "-mlink-builtin-bitcode", "-Xclang", bc, "-S", "--cuda-device-only",
+        os.path.join(hip_build.CSRC, "multi_mma.hip"), "-o", asm]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert r.returncode == 0, r.stdout
+    text = open(asm).read()
+    start = text.index("multi_mma_kernelILi8ELi2ELi8ELi2ELi1EEEvNS0_12MultiMmaArgsE:")
+    body = text[start:text.index("s_endpgm", start)].splitlines()
+    labels = {m.group(1): i for i, l in enumerate(body) for m in [re.match(r"^(\.LBB\d+_\d+):", l)] if m}
+    loops = []
+    for i, l in enumerate(body):
+        m = re.search(r"s_cbranch_\w+\s+(\.LBB\d+_\d+)", l)
+        if m and labels.get(m.group(1), i) < i and any("v_mfma" in x for x in body[labels[m.group(1)]:i]):
+            loops.append((labels[m.group(1)], i))
+    assert len(loops) == 1, loops
+    in_asm, own, compilers = False, [], []
+    for l in body[loops[0][0]:loops[0][1]]:
+        if "#ASMSTART" in l:
+            in_asm = True
+        elif "#ASMEND" in l:
+            in_asm = False
+        elif "vmcnt" in l:
+            (own if in_asm else compilers).append(l.strip())
+    assert own == ["s_waitcnt vmcnt(16)"], own       # two of the ring's three steps in flight, 8 loads each
+    assert compilers == [], compilers
+    assert sum("v_mfma_i32_16x16x64_i8" in l for l in body[loops[0][0]:loops[0][1]]) == 64
