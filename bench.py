@@ -413,7 +413,8 @@ def _also(torch, lib, abi, synth, steps, warmup):
        lhs, rhs, torch.int32, PEAK_INT8_TOPS, "TOP/s")
     # bf16 skinny shapes: M0 in {1, 4, 16}, N = 14336, K = 4096; HBM-bound on the
     # rhs. Three rhs copies are rotated so the 256 MB last-level cache cannot
-    # serve them.
+    # serve them. (The HBM-bound rows are timed over at least 30 launches: theirs
+    # take 20 to 100 us each, and the mean of a handful moves by 2-3 %.)
     nk = 14336 * 4096
     rhs_set = [f16_operand(4, 10 + i, nk, 0.02, bf16=True) for i in range(3)]
     for m0 in (1, 4, 16):
@@ -426,7 +427,7 @@ def _also(torch, lib, abi, synth, steps, warmup):
         def step():
             lib.iree_uk_mmt4d_p(C.byref(ps[state["i"] % 3]))
             state["i"] += 1
-        ms, _ = _time_launches(torch, step, max(steps, 6), warmup)
+        ms, _ = _time_launches(torch, step, max(steps, 30), warmup)
         nbytes = nk * 2 + m0 * 4096 * 2 + 896 * 16 * m0 * 4
         res["mmt4d_bf16_skinny_M%d_N14336_K4096" % m0] = {
             "kernel": lib.iree_uk_mi355x_last_kernel().decode(), "ms": round(ms, 5),
@@ -444,7 +445,7 @@ def _also(torch, lib, abi, synth, steps, warmup):
     def step_narrow():
         lib.iree_uk_mmt4d_p(C.byref(ps[state["i"] % 3]))
         state["i"] += 1
-    ms, _ = _time_launches(torch, step_narrow, max(steps, 6), warmup)
+    ms, _ = _time_launches(torch, step_narrow, max(steps, 30), warmup)
     nbytes = nk * 2 + 4096 * 2 + 896 * 16 * 4
     res["mmt4d_bf16_skinny_x86_tile_1x16x2_N14336_K4096"] = {
         "kernel": lib.iree_uk_mi355x_last_kernel().decode(), "ms": round(ms, 5),
@@ -467,7 +468,7 @@ def _also(torch, lib, abi, synth, steps, warmup):
         def step_i4():
             lib.iree_uk_mmt4d_p(C.byref(ps[state["i"] % 3]))
             state["i"] += 1
-        ms, _ = _time_launches(torch, step_i4, max(steps, 6), warmup)
+        ms, _ = _time_launches(torch, step_i4, max(steps, 30), warmup)
         nbytes = n_i4 * k_i4 // 2 + m0 * k_i4 + n_i4 * m0 * 4
         entry = {"kernel": lib.iree_uk_mi355x_last_kernel().decode(), "ms": round(ms, 5),
                  "value": round(nbytes / ms / 1e6, 1), "unit": "GB/s",
@@ -495,7 +496,7 @@ def _also(torch, lib, abi, synth, steps, warmup):
     def step_vnni():
         lib.iree_uk_mmt4d_p(C.byref(ps[state["i"] % 3]))
         state["i"] += 1
-    ms, _ = _time_launches(torch, step_vnni, max(steps, 6), warmup)
+    ms, _ = _time_launches(torch, step_vnni, max(steps, 30), warmup)
     nbytes = n_i4 * 4096 + 4096 + n_i4 * 4
     entry = {"kernel": lib.iree_uk_mi355x_last_kernel().decode(), "ms": round(ms, 5),
              "value": round(nbytes / ms / 1e6, 1), "unit": "GB/s", "frac_of_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
@@ -534,7 +535,7 @@ def _also(torch, lib, abi, synth, steps, warmup):
             fn, p = ps[state["i"] & 1]
             fn(C.byref(p))
             state["i"] += 1
-        ms, _ = _time_launches(torch, step, max(steps, 6), warmup)
+        ms, _ = _time_launches(torch, step, max(steps, 30), warmup)
         res[name] = {"kernel": lib.iree_uk_mi355x_last_kernel().decode(), "ms": round(ms, 5),
                      "value": round(nbytes / ms / 1e6, 1), "unit": "GB/s",
                      "frac_of_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
@@ -599,7 +600,7 @@ def _also(torch, lib, abi, synth, steps, warmup):
         i = copy_state["i"] & 1
         back[i].copy_(src[i])
         copy_state["i"] += 1
-    ms, _ = _time_launches(torch, copy_step, max(steps, 6), warmup)
+    ms, _ = _time_launches(torch, copy_step, max(steps, 30), warmup)
     res["plain_device_copy_f32_8191x8190_for_comparison"] = {
         "what": "torch.Tensor.copy_ of the same matrix (read + write counted)", "ms": round(ms, 5),
         "value": round(2 * R * Cc * 4 / ms / 1e6, 1), "unit": "GB/s",
@@ -629,7 +630,7 @@ def _also(torch, lib, abi, synth, steps, warmup):
                 if rc != 0:
                     raise RuntimeError("hbm stream probe failed: HIP error %d" % rc)
                 st["i"] += 1
-            ms, _ = _time_launches(torch, stream_step, max(steps, 6), warmup)
+            ms, _ = _time_launches(torch, stream_step, max(steps, 30), warmup)
             best = ms if best is None else min(best, ms)
         moved = stream_bytes * (2 if mode == 2 else 1)
         ceilings[mode_name] = {"ms": round(best, 5), "value": round(moved / best / 1e6, 1), "unit": "GB/s",
@@ -648,7 +649,7 @@ def _also(torch, lib, abi, synth, steps, warmup):
             if rc != 0:
                 raise RuntimeError("hbm stream probe failed: HIP error %d" % rc)
             st["i"] += 1
-        ms, _ = _time_launches(torch, decode_stream_step, max(steps, 6), warmup)
+        ms, _ = _time_launches(torch, decode_stream_step, max(steps, 30), warmup)
         best = ms if best is None else min(best, ms)
     ceilings["read_only_117MB"] = {"ms": round(best, 5), "value": round(decode_bytes / best / 1e6, 1), "unit": "GB/s",
                                    "frac_of_peak": round(decode_bytes / best / 1e6 / PEAK_HBM_GBS, 4)}
@@ -684,7 +685,7 @@ def _also(torch, lib, abi, synth, steps, warmup):
         def step():
             lib.iree_uk_pack_p(C.byref(ps[state["i"] % 3]))
             state["i"] += 1
-        ms, _ = _time_launches(torch, step, max(steps, 6), warmup)
+        ms, _ = _time_launches(torch, step, max(steps, 30), warmup)
         res[name] = {"kernel": lib.iree_uk_mi355x_last_kernel().decode(), "ms": round(ms, 5),
                      "value": round(2.0 * n16 * n16 / ms / 1e6, 1), "unit": "GB/s",
                      "frac_of_peak": round(2.0 * n16 * n16 / ms / 1e6 / PEAK_HBM_GBS, 4)}
