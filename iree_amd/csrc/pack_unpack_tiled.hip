@@ -1029,13 +1029,14 @@ int plan_transposing(Plan* p) {
   return which;
 }
 
-// Workgroups resident per compute unit, for pack of 4-byte elements into more than 128 MiB. A block's LDS image
+// Workgroups resident per compute unit, for 4-byte elements and more than 128 MiB per side. A block's LDS image
 // is 16 to 20 KiB and its four wavefronts let eight workgroups share a unit; with LDS asked for as if the image
-// were 32 KiB, five do, and large f32 matrices pack faster: [8191, 8190] with 16x1 tiles 6.04 -> 6.17 TB/s, with both
-// transposes 5.74 -> 5.83 (six or four workgroups: in between; three or two: 5.0-5.8); over tiles 16x1, 16x16, 8x8,
-// 16x4, 1x16, the four transpose combinations and [2048, 16384] ... [1024, 65536] between -3 and +8 %, +2 % in the
-// mean. Not for unpack (0 to -6 % over the same grid), not for 1- and 2-byte elements (-1 to -19 %), not for
-// matrices the last-level cache holds (4096^2: -1 to -5 %, 3000^2: -2 to -8 %).
+// were 32 KiB, five do, and large f32 matrices move faster: [8191, 8190] with 16x1 tiles pack 6.04 -> 6.17 TB/s, with
+// both transposes 5.74 -> 5.83 (six or four workgroups: in between; three or two: 5.0-5.8), unpack 6.06 -> 6.17. Over
+// tiles 16x1, 8x8, 16x16, the four transpose combinations and [2048, 16384] ... [1024, 65536], buffers rotated
+// so that the last-level cache does not hold them: pack -3 to +8 %, unpack -6 to +12 %, about +2 % in the mean for
+// both. Not for 1- and 2-byte elements (-1 to -19 %) and not for matrices the last-level cache holds (4096^2:
+// -1 to -5 %, 3000^2: -2 to -8 %).
 void limit_resident_blocks(Plan* p) {
   constexpr size_t kLdsAskedFor = 32 * 1024;
   if (p->elem_bytes == 4 && p->args.total_blocks >= 8192 && p->lds_bytes < kLdsAskedFor) p->lds_bytes = kLdsAskedFor;
@@ -1204,6 +1205,7 @@ hipError_t launch_unpack(const UnpackArgs& original, hipStream_t stream, const c
   plan.args.src = a.in;
   plan.args.dst = a.out;
   plan.args.padding_value = 0;
+  limit_resident_blocks(&plan);
   *name = "unpack_tiled";
   if (plan.line_aligned) {
     const dim3 grid(plan.grid), block(256);
