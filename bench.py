@@ -614,18 +614,20 @@ def _also(torch, lib, abi, synth, steps, warmup):
     probe_lib = library.load_bench_probe()
     sink = torch.zeros(4, dtype=torch.int32, device="cuda")
     stream_bytes = R * Cc * 4 // 16 * 16
-    # (vectors in flight per thread, workgroups (0: one pass), blocks an XCD takes at a time)
-    STREAM_SHAPES = ((4, 0, 1), (8, 0, 1), (4, 4096, 1), (8, 2048, 1), (4, 0, 64), (4, 0, 16), (8, 0, 32))
+    # (vectors in flight per thread, workgroups (0: one pass), blocks an XCD takes at a time, workgroups resident
+    # per compute unit (0: as many as fit))
+    STREAM_SHAPES = ((4, 0, 1, 0), (8, 0, 1, 0), (4, 4096, 1, 0), (8, 2048, 1, 0), (4, 0, 64, 0), (4, 0, 16, 0),
+                     (8, 0, 32, 0), (4, 0, 64, 5), (4, 0, 1, 5), (4, 0, 64, 4), (8, 0, 32, 3))
     ceilings = {}
     for mode, mode_name in ((0, "read_only"), (1, "write_only"), (2, "copy")):
         best = None
-        for unroll, grid, xcd_group in STREAM_SHAPES:
+        for unroll, grid, xcd_group, resident in STREAM_SHAPES:
             st = {"i": 0}
 
             def stream_step():
                 i = st["i"] & 1
                 rc = probe_lib.uk_bench_probe_hbm_stream(mode, back[i].data_ptr(), src[i].data_ptr(), stream_bytes, grid,
-                                                         unroll, 1, xcd_group, sink.data_ptr(),
+                                                         unroll, 1, xcd_group, resident, sink.data_ptr(),
                                                          torch.cuda.current_stream().cuda_stream)
                 if rc != 0:
                     raise RuntimeError("hbm stream probe failed: HIP error %d" % rc)
@@ -639,13 +641,14 @@ def _also(torch, lib, abi, synth, steps, warmup):
     # the read-only stream over that many bytes, same rotation.
     decode_bytes = 14336 * 4096 * 2
     best = None
-    for unroll, grid, xcd_group in STREAM_SHAPES:
+    for unroll, grid, xcd_group, resident in STREAM_SHAPES:
         st = {"i": 0}
 
         def decode_stream_step():
             i = st["i"] & 1
             rc = probe_lib.uk_bench_probe_hbm_stream(0, back[i].data_ptr(), src[i].data_ptr(), decode_bytes, grid, unroll, 1,
-                                                     xcd_group, sink.data_ptr(), torch.cuda.current_stream().cuda_stream)
+                                                     xcd_group, resident, sink.data_ptr(),
+                                                     torch.cuda.current_stream().cuda_stream)
             if rc != 0:
                 raise RuntimeError("hbm stream probe failed: HIP error %d" % rc)
             st["i"] += 1
@@ -655,7 +658,7 @@ def _also(torch, lib, abi, synth, steps, warmup):
                                    "frac_of_peak": round(decode_bytes / best / 1e6 / PEAK_HBM_GBS, 4)}
     res["hbm_stream_ceiling"] = dict(
         ceilings, what="plain read / fill / copy kernels over %d bytes, non-temporal 16-byte accesses, "
-                       "two buffer sets rotated; best of seven launch shapes each (with and without blocks dealt to the XCDs in groups); read_only_117MB: the read-only stream over the %d "
+                       "two buffer sets rotated; best of eleven launch shapes each (with and without blocks dealt to the XCDs in groups, with and without a limit on the workgroups resident per compute unit); read_only_117MB: the read-only stream over the %d "
                        "bytes of rhs a matrix-vector launch reads" % (stream_bytes, decode_bytes))
     del src, packed, back
 

@@ -57,23 +57,26 @@ __global__ __launch_bounds__(256) void stream_kernel(v4i32* __restrict__ dst, co
 }
 
 template <int MODE, int UNROLL, bool STREAMING>
-int launch(void* dst, const void* src, long long vectors, int grid_blocks, int xcd_group, void* sink, hipStream_t s) {
+int launch(void* dst, const void* src, long long vectors, int grid_blocks, int xcd_group, int resident, void* sink,
+           hipStream_t s) {
   const long long one_pass = (vectors + 256 * UNROLL - 1) / (256 * UNROLL);
   const unsigned grid = (unsigned)(grid_blocks > 0 && grid_blocks < one_pass ? grid_blocks : one_pass);
-  hipLaunchKernelGGL((stream_kernel<MODE, UNROLL, STREAMING>), dim3(grid), dim3(256), 0, s, (v4i32*)dst,
+  // Workgroup memory the kernel never touches, asked for only to hold the workgroups per compute unit down.
+  const unsigned lds = resident > 0 ? (unsigned)(160 * 1024 / resident < 65536 ? 160 * 1024 / resident : 65536) : 0u;
+  hipLaunchKernelGGL((stream_kernel<MODE, UNROLL, STREAMING>), dim3(grid), dim3(256), lds, s, (v4i32*)dst,
                      (const v4i32*)src, vectors, xcd_group, (int*)sink);
   return (int)hipGetLastError();
 }
 
 template <int MODE>
 int launch_mode(int unroll, int streaming, void* dst, const void* src, long long vectors, int grid_blocks,
-                int xcd_group, void* sink, hipStream_t s) {
-  if (unroll == 4) return streaming ? launch<MODE, 4, true>(dst, src, vectors, grid_blocks, xcd_group, sink, s)
-                                    : launch<MODE, 4, false>(dst, src, vectors, grid_blocks, xcd_group, sink, s);
-  if (unroll == 8) return streaming ? launch<MODE, 8, true>(dst, src, vectors, grid_blocks, xcd_group, sink, s)
-                                    : launch<MODE, 8, false>(dst, src, vectors, grid_blocks, xcd_group, sink, s);
-  if (unroll == 16) return streaming ? launch<MODE, 16, true>(dst, src, vectors, grid_blocks, xcd_group, sink, s)
-                                     : launch<MODE, 16, false>(dst, src, vectors, grid_blocks, xcd_group, sink, s);
+                int xcd_group, int resident, void* sink, hipStream_t s) {
+  if (unroll == 4) return streaming ? launch<MODE, 4, true>(dst, src, vectors, grid_blocks, xcd_group, resident, sink, s)
+                                    : launch<MODE, 4, false>(dst, src, vectors, grid_blocks, xcd_group, resident, sink, s);
+  if (unroll == 8) return streaming ? launch<MODE, 8, true>(dst, src, vectors, grid_blocks, xcd_group, resident, sink, s)
+                                    : launch<MODE, 8, false>(dst, src, vectors, grid_blocks, xcd_group, resident, sink, s);
+  if (unroll == 16) return streaming ? launch<MODE, 16, true>(dst, src, vectors, grid_blocks, xcd_group, resident, sink, s)
+                                     : launch<MODE, 16, false>(dst, src, vectors, grid_blocks, xcd_group, resident, sink, s);
   return (int)hipErrorInvalidValue;
 }
 
@@ -82,17 +85,17 @@ int launch_mode(int unroll, int streaming, void* dst, const void* src, long long
 // mode 0: read `bytes` from src; 1: write `bytes` to dst; 2: copy src -> dst. `bytes` a multiple of 16, buffers
 // 16-byte aligned. `grid_blocks` workgroups of 256 threads (0: one pass over the buffer, i.e. not persistent),
 // `unroll` (4, 8 or 16) vectors in flight per thread, `streaming` != 0: non-temporal accesses, `xcd_group` > 1:
-// blocks dealt to the XCDs in groups of that many.
+// blocks dealt to the XCDs in groups of that many, `resident` > 0: at most that many workgroups per compute unit.
 // Enqueues one launch on `stream` and returns the HIP status; the caller times it and keeps the best variant.
 UK_API int uk_bench_probe_hbm_stream(int mode, void* dst, const void* src, long long bytes, int grid_blocks,
-                                     int unroll, int streaming, int xcd_group, void* sink, void* stream) {
+                                     int unroll, int streaming, int xcd_group, int resident, void* sink, void* stream) {
   if (bytes <= 0 || bytes % 16) return (int)hipErrorInvalidValue;
   const long long vectors = bytes / 16;
   hipStream_t s = (hipStream_t)stream;
   switch (mode) {
-    case 0: return launch_mode<0>(unroll, streaming, dst, src, vectors, grid_blocks, xcd_group, sink, s);
-    case 1: return launch_mode<1>(unroll, streaming, dst, src, vectors, grid_blocks, xcd_group, sink, s);
-    case 2: return launch_mode<2>(unroll, streaming, dst, src, vectors, grid_blocks, xcd_group, sink, s);
+    case 0: return launch_mode<0>(unroll, streaming, dst, src, vectors, grid_blocks, xcd_group, resident, sink, s);
+    case 1: return launch_mode<1>(unroll, streaming, dst, src, vectors, grid_blocks, xcd_group, resident, sink, s);
+    case 2: return launch_mode<2>(unroll, streaming, dst, src, vectors, grid_blocks, xcd_group, resident, sink, s);
     default: return (int)hipErrorInvalidValue;
   }
 }

@@ -83,7 +83,7 @@ def load_bench_probe():
                                                  C.POINTER(C.c_double), C.POINTER(C.c_double)]
         l.uk_bench_probe_matrix_pipe.restype = C.c_int
         l.uk_bench_probe_hbm_stream.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_longlong, C.c_int, C.c_int,
-                                                C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+                                                C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
         l.uk_bench_probe_hbm_stream.restype = C.c_int
         l.uk_bench_probe_mmt4d_timeline.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_longlong, C.c_longlong,
                                                     C.c_longlong, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
