@@ -617,7 +617,8 @@ def _also(torch, lib, abi, synth, steps, warmup):
     # (vectors in flight per thread, workgroups (0: one pass), blocks an XCD takes at a time, workgroups resident
     # per compute unit (0: as many as fit))
     STREAM_SHAPES = ((4, 0, 1, 0), (8, 0, 1, 0), (4, 4096, 1, 0), (8, 2048, 1, 0), (4, 0, 64, 0), (4, 0, 16, 0),
-                     (8, 0, 32, 0), (4, 0, 64, 5), (4, 0, 1, 5), (4, 0, 64, 4), (8, 0, 32, 3))
+                     (8, 0, 32, 0), (4, 0, 64, 5), (4, 0, 1, 5), (4, 0, 64, 4), (8, 0, 32, 3), (1, 0, 1, 0), (1, 0, 64, 0),
+                     (1, 0, 1, 5), (2, 0, 1, 6), (2, 0, 64, 5), (2, 0, 1, 3))
     ceilings = {}
     for mode, mode_name in ((0, "read_only"), (1, "write_only"), (2, "copy")):
         best = None
@@ -658,7 +659,7 @@ def _also(torch, lib, abi, synth, steps, warmup):
                                    "frac_of_peak": round(decode_bytes / best / 1e6 / PEAK_HBM_GBS, 4)}
     res["hbm_stream_ceiling"] = dict(
         ceilings, what="plain read / fill / copy kernels over %d bytes, non-temporal 16-byte accesses, "
-                       "two buffer sets rotated; best of eleven launch shapes each (with and without blocks dealt to the XCDs in groups, with and without a limit on the workgroups resident per compute unit); read_only_117MB: the read-only stream over the %d "
+                       "two buffer sets rotated; best of seventeen launch shapes each (4 to 32 KiB per workgroup, with and without blocks dealt to the XCDs in groups, with and without a limit on the workgroups resident per compute unit); read_only_117MB: the read-only stream over the %d "
                        "bytes of rhs a matrix-vector launch reads" % (stream_bytes, decode_bytes))
     del src, packed, back
 

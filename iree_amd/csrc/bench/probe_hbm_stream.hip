@@ -71,6 +71,10 @@ int launch(void* dst, const void* src, long long vectors, int grid_blocks, int x
 template <int MODE>
 int launch_mode(int unroll, int streaming, void* dst, const void* src, long long vectors, int grid_blocks,
                 int xcd_group, int resident, void* sink, hipStream_t s) {
+  if (unroll == 1) return streaming ? launch<MODE, 1, true>(dst, src, vectors, grid_blocks, xcd_group, resident, sink, s)
+                                    : launch<MODE, 1, false>(dst, src, vectors, grid_blocks, xcd_group, resident, sink, s);
+  if (unroll == 2) return streaming ? launch<MODE, 2, true>(dst, src, vectors, grid_blocks, xcd_group, resident, sink, s)
+                                    : launch<MODE, 2, false>(dst, src, vectors, grid_blocks, xcd_group, resident, sink, s);
   if (unroll == 4) return streaming ? launch<MODE, 4, true>(dst, src, vectors, grid_blocks, xcd_group, resident, sink, s)
                                     : launch<MODE, 4, false>(dst, src, vectors, grid_blocks, xcd_group, resident, sink, s);
   if (unroll == 8) return streaming ? launch<MODE, 8, true>(dst, src, vectors, grid_blocks, xcd_group, resident, sink, s)
@@ -84,7 +88,7 @@ int launch_mode(int unroll, int streaming, void* dst, const void* src, long long
 
 // mode 0: read `bytes` from src; 1: write `bytes` to dst; 2: copy src -> dst. `bytes` a multiple of 16, buffers
 // 16-byte aligned. `grid_blocks` workgroups of 256 threads (0: one pass over the buffer, i.e. not persistent),
-// `unroll` (4, 8 or 16) vectors in flight per thread, `streaming` != 0: non-temporal accesses, `xcd_group` > 1:
+// `unroll` (1, 2, 4, 8 or 16) vectors in flight per thread, `streaming` != 0: non-temporal accesses, `xcd_group` > 1:
 // blocks dealt to the XCDs in groups of that many, `resident` > 0: at most that many workgroups per compute unit.
 // Enqueues one launch on `stream` and returns the HIP status; the caller times it and keeps the best variant.
 UK_API int uk_bench_probe_hbm_stream(int mode, void* dst, const void* src, long long bytes, int grid_blocks,
